@@ -1,0 +1,35 @@
+/*
+ * aclnnMoeInitRoutingV2 — MI355X build.
+ * Replaces: moe/moe_init_routing_v2/op_host/op_api/aclnn_moe_init_routing_v2.h:42-56 (same symbols, same argument order).
+ *
+ * Expands T tokens top-K ways (flat index i = n*K + j over expertIdx[T,K], row-major), sorts the M = T*K flat entries by
+ * expert id with a stable ascending sort, and returns
+ *   expandedRowIdxOut[i]  = destination row of flat entry i (dropless) / e*C + rank or -1 (drop/pad),
+ *   expandedXOut[dst, :]  = x[i / K, :],
+ *   expertTokensCountOrCumsumOut[e] = per-expert count (flag 2) or inclusive cumsum (flag 1), int32.
+ * x dtype: FLOAT, FLOAT16, BF16 as in the reference (moe_init_routing_v2_def.cpp:22-38); INT8 is accepted as an extension so
+ * that already-quantized activations can be routed (a row gather is dtype-agnostic).
+ */
+#ifndef OPS_TRANSFORMER_AMD_ACLNN_MOE_INIT_ROUTING_V2_H_
+#define OPS_TRANSFORMER_AMD_ACLNN_MOE_INIT_ROUTING_V2_H_
+
+#include "acl/acl.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+ACLNN_API aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
+    const aclTensor* x, const aclTensor* expertIdx, int64_t activeNumOptional, int64_t expertCapacityOptional,
+    int64_t expertNumOptional, int64_t dropPadModeOptional, int64_t expertTokensCountOrCumsumFlagOptional,
+    bool expertTokensBeforeCapacityFlagOptional, const aclTensor* expandedXOut, const aclTensor* expandedRowIdxOut,
+    const aclTensor* expertTokensCountOrCumsumOutOptional, const aclTensor* expertTokensBeforeCapacityOutOptional,
+    uint64_t* workspaceSize, aclOpExecutor** executor);
+
+ACLNN_API aclnnStatus aclnnMoeInitRoutingV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
+                                            aclrtStream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

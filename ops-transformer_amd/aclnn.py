@@ -1,0 +1,303 @@
+"""ctypes binding of libcust_opapi.so and Python-level operators mirroring the reference interface.
+
+Each operator follows the reference's two-phase protocol exactly as a C caller would: build ``aclTensor`` descriptors
+over caller-owned device memory, call ``aclnn<Op>GetWorkspaceSize``, allocate the workspace, call ``aclnn<Op>`` on the
+current HIP stream.  A non-zero status raises :class:`AclnnError` carrying the code and ``aclGetRecentErrMsg()``.
+
+There is no fallback: if the shared library is missing, importing an operator fails with instructions to build it.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libcust_opapi.so")
+
+ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32, ACL_INT64, ACL_BF16 = 0, 1, 2, 3, 9, 27
+ACL_FORMAT_ND = 2
+
+ACLNN_SUCCESS = 0
+ACLNN_ERR_PARAM_NULLPTR = 161001
+ACLNN_ERR_PARAM_INVALID = 161002
+ACLNN_ERR_RUNTIME_ERROR = 361001
+
+_DTYPE_CODE = {
+    torch.float32: ACL_FLOAT,
+    torch.float16: ACL_FLOAT16,
+    torch.int8: ACL_INT8,
+    torch.int32: ACL_INT32,
+    torch.int64: ACL_INT64,
+    torch.bfloat16: ACL_BF16,
+}
+
+
+class AclnnError(RuntimeError):
+    def __init__(self, api, code, message):
+        super().__init__("%s failed with status %d: %s" % (api, code, message))
+        self.api = api
+        self.code = code
+        self.message = message
+
+
+def library_path():
+    return _LIB_PATH
+
+
+_lib = None
+
+_VP = ctypes.c_void_p
+_I64 = ctypes.c_int64
+_U64P = ctypes.POINTER(ctypes.c_uint64)
+_VPP = ctypes.POINTER(ctypes.c_void_p)
+
+_PHASE1_SIGNATURES = {
+    "aclnnMoeInitRoutingV2GetWorkspaceSize":
+        [_VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize":
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulV4GetWorkspaceSize":
+        [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _VP, _VP, _U64P, _VPP],
+    "aclnnMoeFinalizeRoutingV2GetWorkspaceSize":
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _U64P, _VPP],
+}
+_PHASE2 = ["aclnnMoeInitRoutingV2", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnMoeFinalizeRoutingV2"]
+
+
+def lib():
+    """The loaded C-ABI library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python ops-transformer_amd/build.py` (hipcc, gfx950). "
+                "There is no CPU or PyTorch fallback for these operators." % _LIB_PATH)
+        l = ctypes.CDLL(_LIB_PATH)
+        for name, sig in _PHASE1_SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.argtypes = sig
+            fn.restype = ctypes.c_int32
+        for name in _PHASE2:
+            fn = getattr(l, name)
+            fn.argtypes = [_VP, ctypes.c_uint64, _VP, _VP]
+            fn.restype = ctypes.c_int32
+        l.aclCreateTensor.argtypes = [ctypes.POINTER(_I64), ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(_I64), _I64,
+                                      ctypes.c_int, ctypes.POINTER(_I64), ctypes.c_uint64, _VP]
+        l.aclCreateTensor.restype = _VP
+        l.aclDestroyTensor.argtypes = [_VP]
+        l.aclCreateTensorList.argtypes = [ctypes.POINTER(_VP), ctypes.c_uint64]
+        l.aclCreateTensorList.restype = _VP
+        l.aclDestroyTensorList.argtypes = [_VP]
+        l.aclDestroyAclOpExecutor.argtypes = [_VP]
+        l.aclGetRecentErrMsg.restype = ctypes.c_char_p
+        _lib = l
+    return _lib
+
+
+def last_error():
+    return lib().aclGetRecentErrMsg().decode("utf-8", "replace")
+
+
+# ------------------------------------------------------------------------------------------------ descriptors
+def create_tensor(shape, dtype_code, data_ptr, strides=None, offset=0, fmt=ACL_FORMAT_ND):
+    """Raw aclCreateTensor; the caller destroys the handle (or hands it to a tensor list)."""
+    n = len(shape)
+    dims = (_I64 * max(n, 1))(*shape)
+    if strides is None:
+        strides = [1] * n
+        for i in range(n - 2, -1, -1):
+            strides[i] = strides[i + 1] * shape[i + 1]
+    st = (_I64 * max(n, 1))(*strides)
+    h = lib().aclCreateTensor(dims, n, dtype_code, st, offset, fmt, dims, n, _VP(data_ptr))
+    if not h:
+        raise MemoryError("aclCreateTensor failed")
+    return h
+
+
+def tensor_of(t):
+    """aclTensor over a torch tensor's memory with its own sizes and strides (no copy)."""
+    if t is None:
+        return None
+    return create_tensor(list(t.shape), _DTYPE_CODE[t.dtype], t.data_ptr(), list(t.stride()))
+
+
+class _Handles:
+    """Owns descriptor handles for the duration of one operator call."""
+
+    def __init__(self):
+        self.tensors = []
+        self.lists = []
+
+    def tensor(self, t):
+        if t is None:
+            return None
+        h = tensor_of(t)
+        self.tensors.append(h)
+        return h
+
+    def tensor_list(self, ts):
+        if ts is None:
+            return None
+        hs = [tensor_of(t) for t in ts]
+        arr = (_VP * max(len(hs), 1))(*hs)
+        h = lib().aclCreateTensorList(arr, len(hs))
+        self.lists.append(h)  # the list owns its tensors
+        return h
+
+    def close(self):
+        l = lib()
+        for h in self.tensors:
+            l.aclDestroyTensor(h)
+        for h in self.lists:
+            l.aclDestroyTensorList(h)
+        self.tensors, self.lists = [], []
+
+
+class Workspace:
+    """A device scratch buffer reused across operator calls; grows to the largest size any call asked for."""
+
+    def __init__(self):
+        self.tensor = None
+
+    def reserve(self, nbytes, device):
+        if self.tensor is None or self.tensor.numel() < nbytes:
+            self.tensor = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        return self.tensor
+
+
+def _stream_ptr():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _run_two_phase(api, args, device, workspace=None):
+    """args: phase-1 arguments without the two trailing out-parameters."""
+    l = lib()
+    ws_size = ctypes.c_uint64(0)
+    executor = ctypes.c_void_p(None)
+    st = getattr(l, api + "GetWorkspaceSize")(*args, ctypes.byref(ws_size), ctypes.byref(executor))
+    if st != ACLNN_SUCCESS:
+        raise AclnnError(api + "GetWorkspaceSize", st, last_error())
+    ws_ptr = None
+    ws_keepalive = None
+    if ws_size.value > 0:
+        if workspace is not None:
+            ws_keepalive = workspace.reserve(ws_size.value, device)
+        else:
+            ws_keepalive = torch.empty(ws_size.value, dtype=torch.uint8, device=device)
+        ws_ptr = ws_keepalive.data_ptr()
+    st = getattr(l, api)(_VP(ws_ptr), ws_size.value, executor, _VP(_stream_ptr()))
+    if st != ACLNN_SUCCESS:
+        raise AclnnError(api, st, last_error())
+    return ws_keepalive
+
+
+def workspace_size(api, args):
+    """Phase 1 only: returns the workspace byte count and releases the executor."""
+    l = lib()
+    ws_size = ctypes.c_uint64(0)
+    executor = ctypes.c_void_p(None)
+    st = getattr(l, api + "GetWorkspaceSize")(*args, ctypes.byref(ws_size), ctypes.byref(executor))
+    if st != ACLNN_SUCCESS:
+        raise AclnnError(api + "GetWorkspaceSize", st, last_error())
+    l.aclDestroyAclOpExecutor(executor)
+    return ws_size.value
+
+
+# ------------------------------------------------------------------------------------------------ operators
+def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_num=0, drop_pad_mode=0,
+                        expert_tokens_count_or_cumsum_flag=0, expert_tokens_before_capacity_flag=False, out=None,
+                        workspace=None):
+    """aclnnMoeInitRoutingV2.  Returns (expanded_x, expanded_row_idx, expert_tokens_count_or_cumsum | None,
+    expert_tokens_before_capacity | None).  ``out`` may carry preallocated outputs in that order."""
+    T, H = x.shape
+    K = expert_idx.shape[1]
+    M = T * K
+    dev = x.device
+    if out is not None:
+        expanded_x, expanded_row_idx, count_out, before_out = out
+    else:
+        if drop_pad_mode == 0:
+            rows = M if active_num == 0 else min(M, active_num)
+            expanded_x = torch.empty((rows, H), dtype=x.dtype, device=dev)
+        else:
+            expanded_x = torch.empty((expert_num, expert_capacity, H), dtype=x.dtype, device=dev)
+        expanded_row_idx = torch.empty((M,), dtype=torch.int32, device=dev)
+        count_out = (torch.empty((expert_num,), dtype=torch.int32, device=dev)
+                     if (drop_pad_mode == 0 and expert_tokens_count_or_cumsum_flag > 0) else None)
+        before_out = (torch.empty((expert_num,), dtype=torch.int32, device=dev)
+                      if (drop_pad_mode == 1 and expert_tokens_before_capacity_flag) else None)
+    h = _Handles()
+    try:
+        args = [h.tensor(x), h.tensor(expert_idx), active_num, expert_capacity, expert_num, drop_pad_mode,
+                expert_tokens_count_or_cumsum_flag, bool(expert_tokens_before_capacity_flag), h.tensor(expanded_x),
+                h.tensor(expanded_row_idx), h.tensor(count_out), h.tensor(before_out)]
+        _run_two_phase("aclnnMoeInitRoutingV2", args, dev, workspace)
+    finally:
+        h.close()
+    return expanded_x, expanded_row_idx, count_out, before_out
+
+
+def grouped_matmul_swiglu_quant(x, weight, group_list, weight_scale, x_scale, bias=None, offset=None, out=None,
+                                workspace=None):
+    """aclnnGroupedMatmulSwigluQuant.  weight is the [E, K, N] view (contiguous, or ``storage.transpose(1, 2)`` over
+    [E, N, K] storage).  Returns (output int8 [M, N/2], output_scale fp32 [M])."""
+    M = x.shape[0]
+    N = weight.shape[2]
+    dev = x.device
+    if out is not None:
+        output, output_scale = out
+    else:
+        output = torch.empty((M, N // 2), dtype=torch.int8, device=dev)
+        output_scale = torch.empty((M,), dtype=torch.float32, device=dev)
+    h = _Handles()
+    try:
+        args = [h.tensor(x), h.tensor(weight), h.tensor(bias), h.tensor(offset), h.tensor(weight_scale),
+                h.tensor(x_scale), h.tensor(group_list), h.tensor(output), h.tensor(output_scale), None]
+        _run_two_phase("aclnnGroupedMatmulSwigluQuant", args, dev, workspace)
+    finally:
+        h.close()
+    return output, output_scale
+
+
+def grouped_matmul_v4(x, weight, bias=None, scale=None, offset=None, antiquant_scale=None, antiquant_offset=None,
+                      per_token_scale=None, group_list=None, activation_input=None, activation_quant_scale=None,
+                      activation_quant_offset=None, split_item=0, group_type=-1, group_list_type=0, act_type=0,
+                      output_dtype=None, out=None, workspace=None):
+    """aclnnGroupedMatmulV4.  x / weight / scale / per_token_scale / out are lists of tensors as in the reference.
+    Returns the list of outputs."""
+    dev = x[0].device
+    if out is None:
+        if output_dtype is None:
+            output_dtype = torch.int32 if scale is None else (
+                torch.bfloat16 if scale[0].dtype == torch.bfloat16 else torch.float16)
+        out = [torch.empty((x[0].shape[0], weight[0].shape[2]), dtype=output_dtype, device=dev)]
+    h = _Handles()
+    try:
+        args = [h.tensor_list(x), h.tensor_list(weight), h.tensor_list(bias), h.tensor_list(scale),
+                h.tensor_list(offset), h.tensor_list(antiquant_scale), h.tensor_list(antiquant_offset),
+                h.tensor_list(per_token_scale), h.tensor(group_list), h.tensor_list(activation_input),
+                h.tensor_list(activation_quant_scale), h.tensor_list(activation_quant_offset), split_item, group_type,
+                group_list_type, act_type, h.tensor_list(out), None, None]
+        _run_two_phase("aclnnGroupedMatmulV4", args, dev, workspace)
+    finally:
+        h.close()
+    return out
+
+
+def moe_finalize_routing_v2(expanded_x, expanded_row_idx, x1=None, x2=None, bias=None, scales=None, expert_idx=None,
+                            drop_pad_mode=0, out=None):
+    """aclnnMoeFinalizeRoutingV2.  Returns out [T, H] in the dtype of expanded_x."""
+    K = 1 if scales is None else scales.shape[1]
+    T = expanded_row_idx.shape[0] // K
+    H = expanded_x.shape[-1]
+    dev = expanded_x.device
+    if out is None:
+        out = torch.empty((T, H), dtype=expanded_x.dtype, device=dev)
+    h = _Handles()
+    try:
+        args = [h.tensor(expanded_x), h.tensor(expanded_row_idx), h.tensor(x1), h.tensor(x2), h.tensor(bias),
+                h.tensor(scales), h.tensor(expert_idx), drop_pad_mode, h.tensor(out)]
+        _run_two_phase("aclnnMoeFinalizeRoutingV2", args, dev)
+    finally:
+        h.close()
+    return out

@@ -1,0 +1,174 @@
+// HIP-backed implementation of the small AscendCL host surface declared in include/acl/acl.h, plus the shared
+// phase-2 driver and the per-thread error text of the aclnn entry points.
+#include "opapi_common.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+namespace {
+thread_local std::string g_lastError;
+
+aclError FromHip(hipError_t e) {
+    if (e == hipSuccess) return ACL_SUCCESS;
+    opapi::SetError("HIP runtime error %d: %s", (int)e, hipGetErrorString(e));
+    return e == hipErrorOutOfMemory ? ACL_ERROR_BAD_ALLOC : ACL_ERROR_RT_FAILURE;
+}
+}  // namespace
+
+namespace opapi {
+
+void SetError(const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_lastError = buf;
+    if (const char* v = std::getenv("OPAPI_LOG_ERRORS")) {
+        if (v[0] != '\0' && v[0] != '0') fprintf(stderr, "[opapi] %s\n", buf);
+    }
+}
+
+void ClearError() { g_lastError.clear(); }
+
+std::string ShapeStr(const aclTensor* t) {
+    if (t == nullptr) return "null";
+    std::string s = "[";
+    for (size_t i = 0; i < t->dims.size(); ++i) {
+        if (i) s += ",";
+        s += std::to_string(t->dims[i]);
+    }
+    return s + "]";
+}
+
+aclnnStatus RunAndRelease(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor, aclrtStream stream) {
+    if (executor == nullptr) {
+        SetError("second-phase call: executor must not be null");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    aclnnStatus st = ACLNN_SUCCESS;
+    if (executor->workspaceBytes > 0 && workspace == nullptr) {
+        SetError("second-phase call: workspace is null but %llu bytes are required",
+                 (unsigned long long)executor->workspaceBytes);
+        st = ACLNN_ERR_PARAM_NULLPTR;
+    } else if (workspaceSize < executor->workspaceBytes) {
+        SetError("second-phase call: workspaceSize %llu is smaller than the required %llu",
+                 (unsigned long long)workspaceSize, (unsigned long long)executor->workspaceBytes);
+        st = ACLNN_ERR_PARAM_INVALID;
+    } else {
+        st = executor->Run(workspace, static_cast<hipStream_t>(stream));
+        if (st == ACLNN_SUCCESS) {
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) {
+                SetError("kernel launch failed: %s", hipGetErrorString(e));
+                st = ACLNN_ERR_RUNTIME_ERROR;
+            }
+        }
+    }
+    delete executor;  // phase 2 consumes the executor
+    return st;
+}
+
+}  // namespace opapi
+
+extern "C" {
+
+aclError aclInit(const char*) { return ACL_SUCCESS; }
+aclError aclFinalize(void) { return ACL_SUCCESS; }
+aclError aclrtSetDevice(int32_t deviceId) { return FromHip(hipSetDevice(deviceId)); }
+aclError aclrtResetDevice(int32_t deviceId) {
+    (void)deviceId;
+    return FromHip(hipDeviceSynchronize());
+}
+aclError aclrtCreateStream(aclrtStream* stream) {
+    if (stream == nullptr) return ACL_ERROR_INVALID_PARAM;
+    hipStream_t s = nullptr;
+    aclError e = FromHip(hipStreamCreate(&s));
+    *stream = s;
+    return e;
+}
+aclError aclrtDestroyStream(aclrtStream stream) { return FromHip(hipStreamDestroy(static_cast<hipStream_t>(stream))); }
+aclError aclrtSynchronizeStream(aclrtStream stream) {
+    return FromHip(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+}
+aclError aclrtMalloc(void** devPtr, size_t size, aclrtMemMallocPolicy) {
+    if (devPtr == nullptr) return ACL_ERROR_INVALID_PARAM;
+    return FromHip(hipMalloc(devPtr, size));
+}
+aclError aclrtFree(void* devPtr) { return FromHip(hipFree(devPtr)); }
+aclError aclrtMemcpy(void* dst, size_t destMax, const void* src, size_t count, aclrtMemcpyKind kind) {
+    if (count > destMax) return ACL_ERROR_INVALID_PARAM;
+    if (count == 0) return ACL_SUCCESS;
+    hipMemcpyKind k = hipMemcpyDefault;
+    switch (kind) {
+        case ACL_MEMCPY_HOST_TO_HOST: k = hipMemcpyHostToHost; break;
+        case ACL_MEMCPY_HOST_TO_DEVICE: k = hipMemcpyHostToDevice; break;
+        case ACL_MEMCPY_DEVICE_TO_HOST: k = hipMemcpyDeviceToHost; break;
+        case ACL_MEMCPY_DEVICE_TO_DEVICE: k = hipMemcpyDeviceToDevice; break;
+    }
+    return FromHip(hipMemcpy(dst, src, count, k));
+}
+aclError aclrtMemset(void* devPtr, size_t maxCount, int32_t value, size_t count) {
+    if (count > maxCount) return ACL_ERROR_INVALID_PARAM;
+    return FromHip(hipMemset(devPtr, value, count));
+}
+
+aclTensor* aclCreateTensor(const int64_t* viewDims, uint64_t viewDimsNum, aclDataType dataType, const int64_t* stride,
+                           int64_t offset, aclFormat format, const int64_t* storageDims, uint64_t storageDimsNum,
+                           void* tensorData) {
+    if ((viewDimsNum > 0 && viewDims == nullptr) || viewDimsNum > 8 || storageDimsNum > 8) return nullptr;
+    aclTensor* t = new (std::nothrow) aclTensor();
+    if (t == nullptr) return nullptr;
+    t->dims.assign(viewDims, viewDims + viewDimsNum);
+    if (stride != nullptr) {
+        t->strides.assign(stride, stride + viewDimsNum);
+    } else {  // contiguous default
+        t->strides.assign(viewDimsNum, 1);
+        for (int i = (int)viewDimsNum - 2; i >= 0; --i) t->strides[i] = t->strides[i + 1] * t->dims[i + 1];
+    }
+    if (storageDims != nullptr) t->storage.assign(storageDims, storageDims + storageDimsNum);
+    t->offset = offset;
+    t->dtype = dataType;
+    t->format = format;
+    t->data = tensorData;
+    return t;
+}
+aclnnStatus aclDestroyTensor(const aclTensor* tensor) {
+    delete tensor;
+    return ACLNN_SUCCESS;
+}
+aclTensorList* aclCreateTensorList(const aclTensor* const* value, uint64_t size) {
+    if (size > 0 && value == nullptr) return nullptr;
+    aclTensorList* l = new (std::nothrow) aclTensorList();
+    if (l == nullptr) return nullptr;
+    l->items.assign(value, value + size);
+    return l;
+}
+aclnnStatus aclDestroyTensorList(const aclTensorList* tensorList) {
+    if (tensorList != nullptr) {
+        for (const aclTensor* t : tensorList->items) delete t;
+        delete tensorList;
+    }
+    return ACLNN_SUCCESS;
+}
+aclIntArray* aclCreateIntArray(const int64_t* value, uint64_t size) {
+    if (size > 0 && value == nullptr) return nullptr;
+    aclIntArray* a = new (std::nothrow) aclIntArray();
+    if (a == nullptr) return nullptr;
+    a->values.assign(value, value + size);
+    return a;
+}
+aclnnStatus aclDestroyIntArray(const aclIntArray* array) {
+    delete array;
+    return ACLNN_SUCCESS;
+}
+aclnnStatus aclDestroyAclOpExecutor(aclOpExecutor* executor) {
+    delete executor;
+    return ACLNN_SUCCESS;
+}
+
+const char* aclGetRecentErrMsg(void) { return g_lastError.c_str(); }
+void ResetCacheThreadLocal(void) { g_lastError.clear(); }
+
+}  // extern "C"

@@ -1,0 +1,503 @@
+// aclnnMoeInitRoutingV2 for gfx950: top-k expansion, stable sort by expert, inverse map, per-expert counts, row gather.
+//
+// Reference behaviour restated (not its structure): moe/moe_init_routing_v2/op_kernel/
+//   moe_v2_sort_one_core.h:64-113, moe_v2_sort_multi_core.h:498-504   stable ascending key/value sort of expert ids
+//   moe_v2_src_to_dst_op.h:92-108                                     expandedRowIdx[order[d]] = d
+//   moe_v2_src_to_dst_with_capacity.h:113-194                         drop/pad: e*C + rank or -1, unused rows zero
+//   moe_v2_expert_token_out.h:125-280                                 per-expert count / cumsum
+//   moe_v2_gather_out.h:87-138                                        expandedX[dst] = x[i / K]
+// Validation follows op_host/moe_init_routing_v2_tiling.cpp:129-283.
+//
+// Design.  Expert ids are small integers, so the merge sort of the reference becomes a stable LSD radix sort whose
+// digit covers all of log2(E) bits in one pass (E <= 2048); larger or unknown id ranges take further passes of the
+// same kernels.  One pass is three launches:
+//   digit_histogram : every wavefront owns a contiguous slice of the flat index range and counts digits into its own
+//                     LDS table, 64 keys a step: a ballot per digit bit yields the lanes holding the same digit, the
+//                     lowest such lane adds popcount(mask) to the table.  No atomics, no inter-wave traffic.
+//   digit_scan      : one workgroup turns the [slice][digit] table into exclusive offsets (down the slices, then across
+//                     digits) and, on the last pass, emits count / cumsum.
+//   digit_scatter   : same traversal; destination = running offset + popcount(mask & lanes below), which keeps equal
+//                     keys in index order (stability).  The last pass writes the inverse map directly.
+// The gather reads each source row once with 16-byte lanes and writes its K destinations.
+#include "opapi_common.h"
+
+#include "aclnnop/aclnn_moe_init_routing_v2.h"
+
+namespace {
+
+constexpr int kWaveSize = 64;
+constexpr int kWavesPerBlock = 4;
+constexpr int kSortThreads = kWaveSize * kWavesPerBlock;
+constexpr int kMaxDigitBits = 11;
+constexpr int kMaxBins = 1 << kMaxDigitBits;
+
+struct SortPass {
+    const int32_t* keysIn;
+    const int32_t* payloadIn;  // nullptr on the first pass: payload is the flat index itself
+    int32_t* keysOut;          // nullptr when no later pass or consumer needs the sorted keys
+    int32_t* payloadOut;       // nullptr on the last pass
+    int32_t* table;            // [numSlices][bins]
+    int32_t* binBase;          // [bins] exclusive offsets of each digit value
+    int32_t* binTotal;         // [bins]
+    int64_t total;             // M
+    int32_t sliceLen;          // keys per wavefront slice (multiple of 64)
+    int32_t numSlices;
+    int32_t shift;
+    int32_t bits;
+    int32_t flipSign;          // 1: the top bit of the digit is the key's sign bit, invert it so negatives sort first
+};
+
+__device__ __forceinline__ uint32_t DigitOf(int32_t key, const SortPass& p) {
+    uint32_t d = (static_cast<uint32_t>(key) >> p.shift) & ((1u << p.bits) - 1u);
+    if (p.flipSign) d ^= 1u << (p.bits - 1);
+    return d;
+}
+
+// Orders this wavefront's LDS accesses: writes made by one lane before the call are seen by every lane after it.
+// The LDS unit executes a wavefront's operations in order, so only the compiler needs constraining.
+__device__ __forceinline__ void WaveSync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Lanes of this wavefront (among `valid` ones) whose digit equals mine.
+__device__ __forceinline__ uint64_t MatchDigit(uint32_t digit, int bits, bool valid) {
+    uint64_t mask = __ballot(valid);
+    for (int b = 0; b < bits; ++b) {
+        const bool bit = (digit >> b) & 1u;
+        const uint64_t bal = __ballot(bit);
+        mask &= bit ? bal : ~bal;
+    }
+    return mask;
+}
+
+__global__ __launch_bounds__(kSortThreads) void DigitHistogramKernel(SortPass p) {
+    __shared__ int32_t tbl[kWavesPerBlock][kMaxBins];
+    const int lane = threadIdx.x % kWaveSize;
+    const int wave = threadIdx.x / kWaveSize;
+    const int bins = 1 << p.bits;
+    const int64_t slice = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + wave;
+    if (slice >= p.numSlices) return;
+    for (int b = lane; b < bins; b += kWaveSize) tbl[wave][b] = 0;
+    WaveSync();
+    const int64_t begin = slice * p.sliceLen;
+    for (int off = 0; off < p.sliceLen; off += kWaveSize) {
+        const int64_t i = begin + off + lane;
+        const bool valid = i < p.total;
+        const uint32_t digit = valid ? DigitOf(p.keysIn[i], p) : 0u;
+        const uint64_t mask = MatchDigit(digit, p.bits, valid);
+        if (valid && lane == __ffsll(static_cast<unsigned long long>(mask)) - 1) tbl[wave][digit] += __popcll(mask);
+        WaveSync();
+    }
+    for (int b = lane; b < bins; b += kWaveSize) p.table[slice * bins + b] = tbl[wave][b];
+}
+
+struct CountOutputs {
+    int32_t* countOrCumsum;   // [expertNum] or nullptr
+    int32_t* beforeCapacity;  // [expertNum] or nullptr
+    int32_t flag;             // 1 cumsum, 2 count (applies to countOrCumsum)
+    int32_t expertNum;
+};
+
+// One workgroup of 1024 threads; each thread owns bins/1024 (1 or 2) digit values.
+__global__ __launch_bounds__(1024) void DigitScanKernel(SortPass p, CountOutputs co) {
+    __shared__ int32_t partial[1024];
+    const int bins = 1 << p.bits;
+    const int perThread = (bins + 1023) / 1024;
+    int32_t totals[2] = {0, 0};
+    for (int j = 0; j < perThread; ++j) {
+        const int b = threadIdx.x * perThread + j;
+        if (b >= bins) break;
+        int32_t run = 0;
+        for (int s = 0; s < p.numSlices; ++s) {
+            const int32_t v = p.table[static_cast<int64_t>(s) * bins + b];
+            p.table[static_cast<int64_t>(s) * bins + b] = run;
+            run += v;
+        }
+        totals[j] = run;
+    }
+    const int32_t mine = totals[0] + totals[1];
+    partial[threadIdx.x] = mine;
+    __syncthreads();
+    // Hillis-Steele inclusive scan over the 1024 per-thread sums
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int32_t add = threadIdx.x >= d ? partial[threadIdx.x - d] : 0;
+        __syncthreads();
+        partial[threadIdx.x] += add;
+        __syncthreads();
+    }
+    int32_t base = partial[threadIdx.x] - mine;
+    for (int j = 0; j < perThread; ++j) {
+        const int b = threadIdx.x * perThread + j;
+        if (b >= bins) break;
+        p.binBase[b] = base;
+        p.binTotal[b] = totals[j];
+        if (b < co.expertNum) {
+            if (co.countOrCumsum != nullptr) co.countOrCumsum[b] = co.flag == 1 ? base + totals[j] : totals[j];
+            if (co.beforeCapacity != nullptr) co.beforeCapacity[b] = totals[j];
+        }
+        base += totals[j];
+    }
+}
+
+struct InverseMap {
+    int32_t* expandedRowIdx;  // nullptr unless this is the last pass
+    int32_t dropPad;          // 1: destination is e*capacity + rank or -1
+    int32_t capacity;
+};
+
+__global__ __launch_bounds__(kSortThreads) void DigitScatterKernel(SortPass p, InverseMap im) {
+    __shared__ int32_t tbl[kWavesPerBlock][kMaxBins];
+    const int lane = threadIdx.x % kWaveSize;
+    const int wave = threadIdx.x / kWaveSize;
+    const int bins = 1 << p.bits;
+    const int64_t slice = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + wave;
+    if (slice >= p.numSlices) return;
+    for (int b = lane; b < bins; b += kWaveSize) tbl[wave][b] = p.table[slice * bins + b] + p.binBase[b];
+    WaveSync();
+    const int64_t begin = slice * p.sliceLen;
+    const uint64_t lanesBelow = (1ull << lane) - 1ull;
+    for (int off = 0; off < p.sliceLen; off += kWaveSize) {
+        const int64_t i = begin + off + lane;
+        const bool valid = i < p.total;
+        const int32_t key = valid ? p.keysIn[i] : 0;
+        const uint32_t digit = valid ? DigitOf(key, p) : 0u;
+        const uint64_t mask = MatchDigit(digit, p.bits, valid);
+        int32_t dst = 0;
+        if (valid) dst = tbl[wave][digit] + __popcll(mask & lanesBelow);
+        WaveSync();
+        if (valid && lane == __ffsll(static_cast<unsigned long long>(mask)) - 1) tbl[wave][digit] += __popcll(mask);
+        WaveSync();
+        if (valid) {
+            const int32_t payload = p.payloadIn != nullptr ? p.payloadIn[i] : static_cast<int32_t>(i);
+            if (p.keysOut != nullptr) p.keysOut[dst] = key;
+            if (p.payloadOut != nullptr) p.payloadOut[dst] = payload;
+            if (im.expandedRowIdx != nullptr) {
+                int32_t row = dst;
+                if (im.dropPad) {
+                    const int32_t rank = dst - p.binBase[digit];
+                    row = rank < im.capacity ? static_cast<int32_t>(digit) * im.capacity + rank : -1;
+                }
+                im.expandedRowIdx[payload] = row;
+            }
+        }
+    }
+}
+
+// Per-expert cumsum / count from fully sorted keys, for id ranges wider than one digit:
+// cumsum[e] = number of sorted keys <= e (upper bound).
+__global__ void CountFromSortedKernel(const int32_t* sortedKeys, int64_t total, CountOutputs co) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= co.expertNum) return;
+    auto upper = [&](int32_t v) {
+        int64_t lo = 0, hi = total;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (sortedKeys[mid] <= v) lo = mid + 1; else hi = mid;
+        }
+        return static_cast<int32_t>(lo);
+    };
+    const int32_t hiCount = upper(e);
+    const int32_t loCount = upper(e - 1);
+    if (co.countOrCumsum != nullptr) co.countOrCumsum[e] = co.flag == 1 ? hiCount : hiCount - loCount;
+    if (co.beforeCapacity != nullptr) co.beforeCapacity[e] = hiCount - loCount;
+}
+
+struct GatherArgs {
+    const char* x;
+    char* expandedX;
+    const int32_t* expandedRowIdx;
+    int64_t rowBytes;
+    int64_t tokens;
+    int32_t topK;
+    int64_t activeRows;  // destinations at or beyond this row are not written
+};
+
+constexpr int kGatherThreads = 256;
+constexpr int kMaxCachedK = 64;
+
+// One workgroup per token: the source row is read once and written to each of its K destinations.
+template <typename Vec>
+__global__ __launch_bounds__(kGatherThreads) void GatherRowsKernel(GatherArgs a) {
+    __shared__ int32_t dsts[kMaxCachedK];
+    const int64_t n = blockIdx.x;
+    const int kCached = a.topK < kMaxCachedK ? a.topK : kMaxCachedK;
+    if (threadIdx.x < kCached) dsts[threadIdx.x] = a.expandedRowIdx[n * a.topK + threadIdx.x];
+    __syncthreads();
+    const int64_t vecs = a.rowBytes / static_cast<int64_t>(sizeof(Vec));
+    const Vec* src = reinterpret_cast<const Vec*>(a.x + n * a.rowBytes);
+    for (int64_t v = threadIdx.x; v < vecs; v += kGatherThreads) {
+        const Vec val = src[v];
+        for (int j = 0; j < a.topK; ++j) {
+            const int64_t d = j < kMaxCachedK ? dsts[j] : a.expandedRowIdx[n * a.topK + j];
+            if (d >= 0 && d < a.activeRows) reinterpret_cast<Vec*>(a.expandedX + d * a.rowBytes)[v] = val;
+        }
+    }
+}
+
+// Drop/pad mode: capacity rows of an expert beyond its (capped) token count hold zeros.
+template <typename Vec>
+__global__ __launch_bounds__(kGatherThreads) void ZeroUnusedCapacityKernel(char* expandedX, const int32_t* binTotal,
+                                                                           int32_t capacity, int64_t rowBytes) {
+    const int64_t row = blockIdx.x;
+    const int32_t e = static_cast<int32_t>(row / capacity);
+    const int32_t c = static_cast<int32_t>(row % capacity);
+    if (c < binTotal[e]) return;
+    const int64_t vecs = rowBytes / static_cast<int64_t>(sizeof(Vec));
+    Vec zero;
+    __builtin_memset(&zero, 0, sizeof(Vec));
+    Vec* dst = reinterpret_cast<Vec*>(expandedX + row * rowBytes);
+    for (int64_t v = threadIdx.x; v < vecs; v += kGatherThreads) dst[v] = zero;
+}
+
+int CeilLog2(int64_t v) {
+    int b = 0;
+    while ((1ll << b) < v) ++b;
+    return b;
+}
+
+class InitRoutingExecutor : public aclOpExecutor {
+   public:
+    // problem
+    const char* x = nullptr;
+    const int32_t* expertIdx = nullptr;
+    char* expandedX = nullptr;
+    int32_t* expandedRowIdx = nullptr;
+    int32_t* countOrCumsum = nullptr;
+    int32_t* beforeCapacity = nullptr;
+    int64_t tokens = 0, topK = 0, rowBytes = 0, total = 0, activeRows = 0;
+    int64_t expertNum = 0, capacity = 0;
+    int dropPad = 0, countFlag = 0;
+    // plan
+    int passes = 1;
+    int bitsPerPass[4] = {0, 0, 0, 0};
+    int keyBits = 0;
+    bool signedRange = false;  // id range unknown: sort all 32 bits, sign-aware
+    int32_t sliceLen = 0, numSlices = 0;
+    uint64_t offKeys[2] = {0, 0}, offPayload[2] = {0, 0}, offTable = 0, offBinBase = 0, offBinTotal = 0;
+
+    void Plan() {
+        if (expertNum > 0) {
+            keyBits = CeilLog2(expertNum);
+            if (keyBits < 1) keyBits = 1;
+        } else {
+            keyBits = 32;
+            signedRange = true;
+        }
+        passes = (keyBits + kMaxDigitBits - 1) / kMaxDigitBits;
+        int left = keyBits;
+        for (int i = 0; i < passes; ++i) {
+            const int remainingPasses = passes - i;
+            bitsPerPass[i] = (left + remainingPasses - 1) / remainingPasses;
+            left -= bitsPerPass[i];
+        }
+        // Slices: at most 1024 so the scan's serial walk stays short; at least 256 keys each.
+        int64_t len = (total + 1023) / 1024;
+        if (len < 256) len = 256;
+        len = (len + kWaveSize - 1) / kWaveSize * kWaveSize;
+        sliceLen = static_cast<int32_t>(len);
+        numSlices = static_cast<int32_t>((total + len - 1) / len);
+        if (numSlices < 1) numSlices = 1;
+
+        uint64_t off = 0;
+        auto take = [&](uint64_t bytes) {
+            const uint64_t o = off;
+            off += opapi::AlignUp(bytes, 256);
+            return o;
+        };
+        const bool needSortedKeys = passes > 1;
+        for (int i = 0; i < 2; ++i) {
+            offKeys[i] = needSortedKeys ? take(static_cast<uint64_t>(total) * 4) : 0;
+            offPayload[i] = passes > 1 ? take(static_cast<uint64_t>(total) * 4) : 0;
+        }
+        offTable = take(static_cast<uint64_t>(numSlices) * kMaxBins * 4);
+        offBinBase = take(kMaxBins * 4);
+        offBinTotal = take(kMaxBins * 4);
+        workspaceBytes = total > 0 ? off : 0;
+    }
+
+    template <typename Vec>
+    void LaunchGather(char* ws, hipStream_t stream) const {
+        if (dropPad) {
+            const int32_t* binTotal = reinterpret_cast<const int32_t*>(ws + offBinTotal);
+            hipLaunchKernelGGL(ZeroUnusedCapacityKernel<Vec>, dim3(static_cast<unsigned>(expertNum * capacity)),
+                               dim3(kGatherThreads), 0, stream, expandedX, binTotal, static_cast<int32_t>(capacity),
+                               rowBytes);
+        }
+        GatherArgs g{x, expandedX, expandedRowIdx, rowBytes, tokens, static_cast<int32_t>(topK),
+                     dropPad ? expertNum * capacity : activeRows};
+        hipLaunchKernelGGL(GatherRowsKernel<Vec>, dim3(static_cast<unsigned>(tokens)), dim3(kGatherThreads), 0, stream,
+                           g);
+    }
+
+    aclnnStatus Run(void* workspace, hipStream_t stream) override {
+        if (total == 0) return ACLNN_SUCCESS;
+        char* ws = static_cast<char*>(workspace);
+        const unsigned sortBlocks = static_cast<unsigned>((numSlices + kWavesPerBlock - 1) / kWavesPerBlock);
+        int shift = 0;
+        const int32_t* keysIn = expertIdx;
+        const int32_t* payloadIn = nullptr;
+        for (int pass = 0; pass < passes; ++pass) {
+            const bool last = pass == passes - 1;
+            SortPass p{};
+            p.keysIn = keysIn;
+            p.payloadIn = payloadIn;
+            p.keysOut = passes > 1 ? reinterpret_cast<int32_t*>(ws + offKeys[pass & 1]) : nullptr;
+            p.payloadOut = last ? nullptr : reinterpret_cast<int32_t*>(ws + offPayload[pass & 1]);
+            p.table = reinterpret_cast<int32_t*>(ws + offTable);
+            p.binBase = reinterpret_cast<int32_t*>(ws + offBinBase);
+            p.binTotal = reinterpret_cast<int32_t*>(ws + offBinTotal);
+            p.total = total;
+            p.sliceLen = sliceLen;
+            p.numSlices = numSlices;
+            p.shift = shift;
+            p.bits = bitsPerPass[pass];
+            p.flipSign = (signedRange && last) ? 1 : 0;
+            CountOutputs co{nullptr, nullptr, countFlag, static_cast<int32_t>(expertNum)};
+            if (last && passes == 1) {
+                co.countOrCumsum = countOrCumsum;
+                co.beforeCapacity = beforeCapacity;
+            }
+            InverseMap im{last ? expandedRowIdx : nullptr, dropPad, static_cast<int32_t>(capacity)};
+            hipLaunchKernelGGL(DigitHistogramKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p);
+            hipLaunchKernelGGL(DigitScanKernel, dim3(1), dim3(1024), 0, stream, p, co);
+            hipLaunchKernelGGL(DigitScatterKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p, im);
+            keysIn = p.keysOut;
+            payloadIn = p.payloadOut;
+            shift += bitsPerPass[pass];
+        }
+        if (passes > 1 && (countOrCumsum != nullptr || beforeCapacity != nullptr)) {
+            CountOutputs co{countOrCumsum, beforeCapacity, countFlag, static_cast<int32_t>(expertNum)};
+            const unsigned blocks = static_cast<unsigned>((expertNum + 255) / 256);
+            hipLaunchKernelGGL(CountFromSortedKernel, dim3(blocks), dim3(256), 0, stream, keysIn, total, co);
+        }
+        if (rowBytes > 0 && tokens > 0) {
+            const uintptr_t align = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(expandedX) |
+                                    static_cast<uintptr_t>(rowBytes);
+            if (align % 16 == 0) LaunchGather<uint4>(ws, stream);
+            else if (align % 4 == 0) LaunchGather<uint32_t>(ws, stream);
+            else if (align % 2 == 0) LaunchGather<uint16_t>(ws, stream);
+            else LaunchGather<uint8_t>(ws, stream);
+        }
+        return ACLNN_SUCCESS;
+    }
+};
+
+}  // namespace
+
+extern "C" aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
+    const aclTensor* x, const aclTensor* expertIdx, int64_t activeNum, int64_t expertCapacity, int64_t expertNum,
+    int64_t dropPadMode, int64_t expertTokensCountOrCumsumFlag, bool expertTokensBeforeCapacityFlag,
+    const aclTensor* expandedXOut, const aclTensor* expandedRowIdxOut, const aclTensor* expertTokensCountOrCumsumOut,
+    const aclTensor* expertTokensBeforeCapacityOut, uint64_t* workspaceSize, aclOpExecutor** executor) {
+    using namespace opapi;
+    ClearError();
+    OPAPI_CHECK_NOTNULL(x, "x");
+    OPAPI_CHECK_NOTNULL(expertIdx, "expertIdx");
+    OPAPI_CHECK_NOTNULL(expandedXOut, "expandedXOut");
+    OPAPI_CHECK_NOTNULL(expandedRowIdxOut, "expandedRowIdxOut");
+    OPAPI_CHECK_NOTNULL(workspaceSize, "workspaceSize");
+    OPAPI_CHECK_NOTNULL(executor, "executor");
+
+    constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;
+    OPAPI_CHECK(x->dtype == ACL_FLOAT || x->dtype == ACL_FLOAT16 || x->dtype == ACL_BF16 || x->dtype == ACL_INT8, kInvalid,
+                "x dtype %d is not supported (FLOAT, FLOAT16, BF16, INT8)", (int)x->dtype);
+    OPAPI_CHECK(expertIdx->dtype == ACL_INT32, kInvalid, "expertIdx must be INT32");
+    OPAPI_CHECK(expandedXOut->dtype == x->dtype, kInvalid, "expandedXOut dtype must equal x dtype");
+    OPAPI_CHECK(expandedRowIdxOut->dtype == ACL_INT32, kInvalid, "expandedRowIdxOut must be INT32");
+    OPAPI_CHECK(x->dims.size() == 2, kInvalid, "The dim number of x should be 2.");
+    OPAPI_CHECK(expertIdx->dims.size() == 2, kInvalid, "The dim number of expertIdx should be 2.");
+    OPAPI_CHECK(x->dims[0] == expertIdx->dims[0], kInvalid, "The first dim of x and expertIdx should be equal.");
+    OPAPI_CHECK(activeNum >= 0, kInvalid, "The activeNum cannot be less than 0.");
+    OPAPI_CHECK(expertCapacity >= 0, kInvalid, "The expertCapacity cannot be less than 0.");
+    OPAPI_CHECK(expertNum >= 0, kInvalid, "The expertNum cannot be less than 0.");
+    OPAPI_CHECK(dropPadMode == 0 || dropPadMode == 1, kInvalid, "The dropPadMode should be 0 or 1.");
+    OPAPI_CHECK(!(dropPadMode > 0 && (expertCapacity < 1 || expertNum < 1)), kInvalid,
+                "The expertCapacity and expertNum should be greater than 0 when dropPadMode is 1");
+    OPAPI_CHECK(expertTokensCountOrCumsumFlag >= 0 && expertTokensCountOrCumsumFlag <= 2, kInvalid,
+                "The expertTokensCountOrCumsumFlag should be 0, 1 or 2.");
+    OPAPI_CHECK(!(expertTokensCountOrCumsumFlag > 0 && expertNum <= 0), kInvalid,
+                "The expertNum should be greater than 0 when expertTokensCountOrCumsumFlag is greater than 0");
+    OPAPI_CHECK(!(dropPadMode > 0 && expertCapacity > x->dims[0]), kInvalid,
+                "The first dim of x cannot be less than expertCapacity");
+    OPAPI_CHECK(!(dropPadMode > 0 && expertNum > kMaxBins), kInvalid,
+                "dropPadMode 1 supports at most %d experts in this build", kMaxBins);
+    // drop/pad never emits count-or-cumsum; dropless never emits before-capacity counts
+    int64_t countFlag = dropPadMode == 1 ? 0 : expertTokensCountOrCumsumFlag;
+    bool beforeFlag = dropPadMode == 1 ? expertTokensBeforeCapacityFlag : false;
+
+    const int64_t tokens = x->dims[0], cols = x->dims[1], topK = expertIdx->dims[1];
+    const int64_t total = tokens * topK;
+    OPAPI_CHECK(total < (1ll << 31), kInvalid, "tokens * topK = %lld does not fit int32 row indices", (long long)total);
+    int64_t activeRows = total;
+    if (dropPadMode > 0) {
+        OPAPI_CHECK(expandedXOut->dims.size() == 3, kInvalid, "The dim number of expandedX should be 3.");
+        OPAPI_CHECK(expandedXOut->dims[0] == expertNum, kInvalid, "The first dim of expandedX should be %lld.",
+                    (long long)expertNum);
+        OPAPI_CHECK(expandedXOut->dims[1] == expertCapacity, kInvalid, "The second dim of expandedX should be %lld.",
+                    (long long)expertCapacity);
+        OPAPI_CHECK(expandedXOut->dims[2] == cols, kInvalid, "The third dim of expandedX should be %lld.", (long long)cols);
+        OPAPI_CHECK(expertNum * expertCapacity < (1ll << 31), kInvalid, "expertNum * expertCapacity does not fit int32");
+    } else {
+        activeRows = activeNum == 0 ? total : (activeNum < total ? activeNum : total);
+        OPAPI_CHECK(expandedXOut->dims.size() == 2, kInvalid, "The dim number of expandedX should be 2.");
+        OPAPI_CHECK(expandedXOut->dims[0] == activeRows, kInvalid, "The first dim of expandedX should be %lld.",
+                    (long long)activeRows);
+        OPAPI_CHECK(expandedXOut->dims[1] == cols, kInvalid, "The second dim of expandedX should be %lld.", (long long)cols);
+    }
+    OPAPI_CHECK(expandedRowIdxOut->dims.size() == 1, kInvalid, "The dim number of expandedRowIdx should be 1.");
+    OPAPI_CHECK(expandedRowIdxOut->dims[0] == total, kInvalid, "The first dim of expandedRowIdx should be %lld.",
+                (long long)total);
+    auto checkTokenCount = [&](const aclTensor* t, const char* name) -> aclnnStatus {
+        OPAPI_CHECK(t != nullptr, ACLNN_ERR_PARAM_NULLPTR, "%s must not be null when its flag is set", name);
+        OPAPI_CHECK(t->dtype == ACL_INT32, kInvalid, "%s must be INT32", name);
+        OPAPI_CHECK(t->dims.size() == 1, kInvalid, "The dim number of %s should be 1.", name);
+        OPAPI_CHECK(t->dims[0] == expertNum, kInvalid, "The first dim of %s should be %lld.", name, (long long)expertNum);
+        OPAPI_CHECK(IsContiguous(t), kInvalid, "%s must be contiguous", name);
+        return ACLNN_SUCCESS;
+    };
+    if (countFlag != 0) {
+        aclnnStatus st = checkTokenCount(expertTokensCountOrCumsumOut, "expertTokensCountOrCumsum");
+        if (st != ACLNN_SUCCESS) return st;
+    }
+    if (beforeFlag) {
+        aclnnStatus st = checkTokenCount(expertTokensBeforeCapacityOut, "expertTokensBeforeCapacity");
+        if (st != ACLNN_SUCCESS) return st;
+    }
+    OPAPI_CHECK(IsContiguous(x) && IsContiguous(expertIdx) && IsContiguous(expandedXOut) && IsContiguous(expandedRowIdxOut),
+                kInvalid, "x, expertIdx, expandedXOut and expandedRowIdxOut must be contiguous");
+    if (total > 0) {
+        OPAPI_CHECK(expertIdx->data != nullptr && expandedRowIdxOut->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
+                    "expertIdx / expandedRowIdxOut carry no device memory");
+        OPAPI_CHECK(cols == 0 || (x->data != nullptr && expandedXOut->data != nullptr), ACLNN_ERR_PARAM_NULLPTR,
+                    "x / expandedXOut carry no device memory");
+    }
+
+    auto* ex = new (std::nothrow) InitRoutingExecutor();
+    OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
+    ex->x = DataPtr(x);
+    ex->expertIdx = reinterpret_cast<const int32_t*>(DataPtr(expertIdx));
+    ex->expandedX = DataPtr(expandedXOut);
+    ex->expandedRowIdx = reinterpret_cast<int32_t*>(DataPtr(expandedRowIdxOut));
+    ex->countOrCumsum = countFlag != 0 ? reinterpret_cast<int32_t*>(DataPtr(expertTokensCountOrCumsumOut)) : nullptr;
+    ex->beforeCapacity = beforeFlag ? reinterpret_cast<int32_t*>(DataPtr(expertTokensBeforeCapacityOut)) : nullptr;
+    ex->tokens = tokens;
+    ex->topK = topK;
+    ex->rowBytes = cols * ElemSize(x->dtype);
+    ex->total = total;
+    ex->activeRows = activeRows;
+    ex->expertNum = expertNum;
+    ex->capacity = expertCapacity;
+    ex->dropPad = static_cast<int>(dropPadMode);
+    ex->countFlag = static_cast<int>(countFlag);
+    ex->Plan();
+    *workspaceSize = ex->workspaceBytes;
+    *executor = ex;
+    return ACLNN_SUCCESS;
+}
+
+extern "C" aclnnStatus aclnnMoeInitRoutingV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
+                                             aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
+}

@@ -1,0 +1,112 @@
+// Shared host-side plumbing of the aclnn C-ABI: descriptor objects, executors, error reporting, argument checks.
+// Every aclnn entry point is two-phase (docs/context/两段式接口.md:5-20 in the reference): phase 1 validates, plans and
+// returns a heap executor plus the workspace byte count; phase 2 enqueues on the caller's stream and consumes the executor.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "acl/acl.h"
+
+struct aclTensor {
+    std::vector<int64_t> dims;     // view shape
+    std::vector<int64_t> strides;  // in elements
+    std::vector<int64_t> storage;  // storage shape
+    int64_t offset = 0;            // in elements
+    aclDataType dtype = ACL_DT_UNDEFINED;
+    aclFormat format = ACL_FORMAT_ND;
+    void* data = nullptr;
+};
+
+struct aclTensorList {
+    std::vector<const aclTensor*> items;
+};
+
+struct aclIntArray {
+    std::vector<int64_t> values;
+};
+
+struct aclOpExecutor {
+    uint64_t workspaceBytes = 0;
+    virtual ~aclOpExecutor() = default;
+    // Enqueue all kernels of the op on `stream`; must not synchronise with the host.
+    virtual aclnnStatus Run(void* workspace, hipStream_t stream) = 0;
+};
+
+namespace opapi {
+
+void SetError(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void ClearError();
+
+// Phase-2 body shared by all ops: argument checks, Run, launch-error check, executor release.
+aclnnStatus RunAndRelease(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor, aclrtStream stream);
+
+inline int64_t ElemSize(aclDataType dt) {
+    switch (dt) {
+        case ACL_FLOAT: case ACL_INT32: case ACL_UINT32: return 4;
+        case ACL_FLOAT16: case ACL_BF16: case ACL_INT16: case ACL_UINT16: return 2;
+        case ACL_INT8: case ACL_UINT8: case ACL_BOOL: return 1;
+        case ACL_INT64: case ACL_UINT64: case ACL_DOUBLE: return 8;
+        default: return 0;
+    }
+}
+
+inline int64_t Numel(const aclTensor* t) {
+    int64_t n = 1;
+    for (int64_t d : t->dims) n *= d;
+    return n;
+}
+
+inline bool IsEmpty(const aclTensor* t) { return t == nullptr || Numel(t) == 0; }
+
+// Row-major contiguous view (dims of extent 1 may carry any stride).
+inline bool IsContiguous(const aclTensor* t) {
+    int64_t expect = 1;
+    for (int i = (int)t->dims.size() - 1; i >= 0; --i) {
+        if (t->dims[i] != 1 && t->strides[i] != expect) return false;
+        expect *= t->dims[i];
+    }
+    return true;
+}
+
+// The last two view dims are a transpose of contiguous storage: strides (.., 1, dim[-2]).  This is how the reference
+// recognises a transposed weight (gmm/grouped_matmul/op_host/op_api/aclnn_grouped_matmul_util.cpp:20-32).
+inline bool IsLastTwoDimsTransposed(const aclTensor* t) {
+    const int n = (int)t->dims.size();
+    if (n < 2) return false;
+    const int64_t d1 = t->dims[n - 1], d2 = t->dims[n - 2];
+    if (t->strides[n - 2] != 1 || t->strides[n - 1] != d2) return false;
+    int64_t expect = d1 * d2;
+    for (int i = n - 3; i >= 0; --i) {
+        if (t->dims[i] != 1 && t->strides[i] != expect) return false;
+        expect *= t->dims[i];
+    }
+    // a [.., 1, 1] tail is both; call it not transposed
+    return !(d1 == 1 && d2 == 1);
+}
+
+inline char* DataPtr(const aclTensor* t) {
+    return t == nullptr ? nullptr : static_cast<char*>(t->data) + t->offset * ElemSize(t->dtype);
+}
+
+inline uint64_t AlignUp(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+std::string ShapeStr(const aclTensor* t);
+
+}  // namespace opapi
+
+#define OPAPI_CHECK(cond, code, ...)            \
+    do {                                        \
+        if (!(cond)) {                          \
+            ::opapi::SetError(__VA_ARGS__);     \
+            return (code);                      \
+        }                                       \
+    } while (0)
+
+#define OPAPI_CHECK_NOTNULL(ptr, name) \
+    OPAPI_CHECK((ptr) != nullptr, ACLNN_ERR_PARAM_NULLPTR, "%s: argument %s must not be null", __func__, name)

@@ -1,0 +1,78 @@
+"""The quantized MoE expert FFN as a chain of the four aclnn operators (the caller side of the path).
+
+    aclnnMoeInitRoutingV2 -> aclnnGroupedMatmulSwigluQuant -> aclnnGroupedMatmulV4 -> aclnnMoeFinalizeRoutingV2
+
+The reference has no in-repo code that chains them; real callers (torch_npu, vLLM-Ascend) do what ``forward`` does.
+Glue between the operators:
+  * activations arrive already quantized per token (int8 rows + fp32 scale); the rows are routed with the INT8
+    extension of MoeInitRoutingV2 and the per-token scales are routed by a second MoeInitRoutingV2 call on the
+    [T, 1] fp32 scale column (a row gather commutes with per-row quantization bit-exactly);
+  * routing emits an int32 cumsum; both GEMM operators of this build accept it directly;
+  * MoeFinalizeRoutingV2 is called with dropPadMode 2 because MoeInitRoutingV2 emits the row arrangement
+    (expandedRowIdx[n*K + k]).
+"""
+import torch
+
+from . import aclnn
+
+
+class MoeFfnW8A8:
+    """Expert weights resident on one GPU plus preallocated intermediates for a fixed (tokens, top_k).
+
+    w13: int8 storage [E, 2I, H]  (gate/up projection, K-contiguous: row n holds the H weights of output channel n;
+         channels [0, I) are the activated half, [I, 2I) the linear half)
+    w13_scale: fp32 [E, 2I]
+    w2:  int8 storage [E, H, I]   (down projection, K-contiguous)
+    w2_scale:  fp32 or bf16 [E, H]
+    The operators see the reference layout [E, K, N] through transposed views of this storage.
+    """
+
+    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16):
+        assert w13.dtype == torch.int8 and w2.dtype == torch.int8
+        self.w13_view = w13.transpose(1, 2)  # [E, H, 2I]
+        self.w2_view = w2.transpose(1, 2)    # [E, I, H]
+        self.w13_scale = w13_scale
+        self.w2_scale = w2_scale
+        self.num_experts = w13.shape[0]
+        self.hidden = w13.shape[2]
+        self.inter = w13.shape[1] // 2
+        self.out_dtype = out_dtype
+        self.device = w13.device
+        self._buf_key = None
+
+    def _buffers(self, T, K):
+        if self._buf_key == (T, K):
+            return
+        dev, M, H, I, E = self.device, T * K, self.hidden, self.inter, self.num_experts
+        self.expanded_x = torch.empty((M, H), dtype=torch.int8, device=dev)
+        self.expanded_row_idx = torch.empty((M,), dtype=torch.int32, device=dev)
+        self.cumsum = torch.empty((E,), dtype=torch.int32, device=dev)
+        self.expanded_scale = torch.empty((M, 1), dtype=torch.float32, device=dev)
+        self.row_idx_scratch = torch.empty((M,), dtype=torch.int32, device=dev)
+        self.h = torch.empty((M, I), dtype=torch.int8, device=dev)
+        self.h_scale = torch.empty((M,), dtype=torch.float32, device=dev)
+        self.y = torch.empty((M, H), dtype=self.out_dtype, device=dev)
+        self.out = torch.empty((T, H), dtype=self.out_dtype, device=dev)
+        # one workspace shared by the chain; it grows to the largest phase-1 request on the first pass
+        self.workspace = aclnn.Workspace()
+        self._buf_key = (T, K)
+
+    def forward(self, xq, x_scale, topk_idx, topk_weight):
+        """xq int8 [T, H]; x_scale fp32 [T]; topk_idx int32 [T, K]; topk_weight fp32/bf16 [T, K] -> out [T, H]."""
+        T, K = topk_idx.shape
+        self._buffers(T, K)
+        E = self.num_experts
+        aclnn.moe_init_routing_v2(xq, topk_idx, 0, 0, E, 0, 1, False,
+                                  out=(self.expanded_x, self.expanded_row_idx, self.cumsum, None),
+                                  workspace=self.workspace)
+        aclnn.moe_init_routing_v2(x_scale.view(T, 1), topk_idx, 0, 0, E, 0, 0, False,
+                                  out=(self.expanded_scale, self.row_idx_scratch, None, None),
+                                  workspace=self.workspace)
+        aclnn.grouped_matmul_swiglu_quant(self.expanded_x, self.w13_view, self.cumsum, self.w13_scale,
+                                          self.expanded_scale.view(T * K), out=(self.h, self.h_scale),
+                                          workspace=self.workspace)
+        aclnn.grouped_matmul_v4([self.h], [self.w2_view], scale=[self.w2_scale], per_token_scale=[self.h_scale],
+                                group_list=self.cumsum, split_item=3, group_type=0, group_list_type=0, act_type=0,
+                                out=[self.y], workspace=self.workspace)
+        aclnn.moe_finalize_routing_v2(self.y, self.expanded_row_idx, scales=topk_weight, drop_pad_mode=2, out=self.out)
+        return self.out

@@ -1,0 +1,207 @@
+"""CPU oracle for the quantized MoE expert-FFN path — TEST INFRASTRUCTURE, never part of the product path.
+
+Thin numpy/ctypes front end over ``liboracle.so`` (built from ``moe_ffn_oracle.c`` by ``make -C oracle``).
+Only the test-suite, the smoke check and the benchmark's ``cpu_baseline`` leg import this module; the
+shipped library and its Python host layer never do.
+
+Half-precision tensors travel as ``uint16`` numpy arrays holding the raw bits (dtype code 1 = fp16, 27 = bf16,
+0 = fp32, the ge::DataType numbering the reference uses).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+DT_F32, DT_F16, DT_BF16 = 0, 1, 27
+
+
+def build(force=False):
+    """Compile the oracle with gcc (seconds)."""
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(
+            os.path.join(_HERE, "moe_ffn_oracle.c")):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.oracle_moe_init_routing_v2.restype = ctypes.c_int
+        _lib.oracle_num_threads.restype = ctypes.c_int
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype=None):
+    if a is None:
+        return None
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def num_threads():
+    return int(lib().oracle_num_threads())
+
+
+# ----------------------------------------------------------------------------------------------- casts
+def f32_to_bf16_bits(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, np.uint16)
+    lib().oracle_f32_to_bf16(_p(a), _p(out), ctypes.c_int64(a.size))
+    return out
+
+
+def f32_to_f16_bits(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, np.uint16)
+    lib().oracle_f32_to_f16(_p(a), _p(out), ctypes.c_int64(a.size))
+    return out
+
+
+def f16_bits_to_f32(a):
+    a = _c(a, np.uint16)
+    out = np.empty(a.shape, np.float32)
+    lib().oracle_f16_to_f32(_p(a), _p(out), ctypes.c_int64(a.size))
+    return out
+
+
+def bf16_bits_to_f32(a):
+    a = _c(a, np.uint16)
+    out = np.empty(a.shape, np.float32)
+    lib().oracle_bf16_to_f32(_p(a), _p(out), ctypes.c_int64(a.size))
+    return out
+
+
+def to_f32(a, dtype_code):
+    if dtype_code == DT_F32:
+        return np.asarray(a, np.float32)
+    return f16_bits_to_f32(a) if dtype_code == DT_F16 else bf16_bits_to_f32(a)
+
+
+def from_f32(a, dtype_code):
+    if dtype_code == DT_F32:
+        return np.asarray(a, np.float32)
+    return f32_to_f16_bits(a) if dtype_code == DT_F16 else f32_to_bf16_bits(a)
+
+
+# ----------------------------------------------------------------------------------------------- routing
+def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_num=0, drop_pad_mode=0,
+                        count_flag=0, before_capacity_flag=False):
+    """x: [T, H] array of any fixed-size dtype (rows are copied as bytes); expert_idx: int32 [T, K].
+
+    Returns (expandedX, expandedRowIdx, countOrCumsum | None, beforeCapacity | None)."""
+    x = _c(x)
+    expert_idx = _c(expert_idx, np.int32)
+    T, K = expert_idx.shape
+    H = x.shape[1]
+    M = T * K
+    row_bytes = H * x.dtype.itemsize
+    if drop_pad_mode == 0:
+        rows = M if active_num == 0 else min(M, active_num)
+        ex = np.zeros((rows, H), x.dtype)
+    else:
+        ex = np.zeros((expert_num, expert_capacity, H), x.dtype)
+    idx = np.full((M,), -7, np.int32)
+    eff_count_flag = 0 if drop_pad_mode == 1 else count_flag
+    eff_before = bool(before_capacity_flag) and drop_pad_mode == 1
+    cnt = np.zeros((expert_num,), np.int32) if eff_count_flag else None
+    bef = np.zeros((expert_num,), np.int32) if eff_before else None
+    rc = lib().oracle_moe_init_routing_v2(
+        _p(x), ctypes.c_int64(row_bytes), _p(expert_idx), ctypes.c_int64(T), ctypes.c_int64(K),
+        ctypes.c_int64(active_num), ctypes.c_int64(expert_capacity), ctypes.c_int64(expert_num),
+        ctypes.c_int64(drop_pad_mode), ctypes.c_int64(count_flag), ctypes.c_int(1 if before_capacity_flag else 0),
+        _p(ex), _p(idx), _p(cnt), _p(bef))
+    if rc != 0:
+        raise ValueError("expert id outside [0, expert_num)")
+    return ex, idx, cnt, bef
+
+
+# ----------------------------------------------------------------------------------------------- GEMMs
+def _gemm_common(x, w, w_trans, group_list, rows):
+    x = _c(x, np.int8)
+    w = _c(w, np.int8)
+    M, K = x.shape
+    if w_trans:
+        G, N, K2 = w.shape
+    else:
+        G, K2, N = w.shape
+    assert K2 == K, (w.shape, x.shape)
+    gl = _c(group_list, np.int64)
+    assert gl.shape[0] <= G
+    rows_a = None if rows is None else _c(rows, np.int64)
+    cnt = M if rows is None else rows_a.shape[0]
+    return x, w, M, K, N, gl, rows_a, cnt
+
+
+def grouped_matmul_i32(x, w, group_list, list_type=0, w_trans=False, rows=None):
+    """Raw int32 accumulators. w: int8 [G, K, N] (w_trans False) or [G, N, K] storage (w_trans True)."""
+    x, w, M, K, N, gl, rows_a, cnt = _gemm_common(x, w, w_trans, group_list, rows)
+    out = np.zeros((cnt, N), np.int32)
+    lib().oracle_grouped_matmul_i32(_p(x), _p(w), ctypes.c_int(int(w_trans)), ctypes.c_int64(M), ctypes.c_int64(K),
+                                    ctypes.c_int64(N), ctypes.c_int64(gl.shape[0]), _p(gl), ctypes.c_int64(list_type),
+                                    _p(rows_a), ctypes.c_int64(cnt), _p(out))
+    return out
+
+
+def grouped_matmul_swiglu_quant(x, w, w_scale, x_scale, group_list, w_trans=False, w_scale_dtype=DT_F32, rows=None,
+                                want_s=False):
+    """Returns (y int8 [cnt, N/2], yScale fp32 [cnt]) and, with want_s, also S fp32 [cnt, N/2]."""
+    x, w, M, K, N, gl, rows_a, cnt = _gemm_common(x, w, w_trans, group_list, rows)
+    ws = _c(w_scale, np.float32 if w_scale_dtype == DT_F32 else np.uint16)
+    xs = _c(x_scale, np.float32)
+    y = np.zeros((cnt, N // 2), np.int8)
+    ys = np.zeros((cnt,), np.float32)
+    s = np.zeros((cnt, N // 2), np.float32) if want_s else None
+    lib().oracle_grouped_matmul_swiglu_quant(
+        _p(x), _p(w), ctypes.c_int(int(w_trans)), _p(ws), ctypes.c_int(w_scale_dtype), _p(xs), ctypes.c_int64(M),
+        ctypes.c_int64(K), ctypes.c_int64(N), ctypes.c_int64(gl.shape[0]), _p(gl), _p(rows_a), ctypes.c_int64(cnt),
+        _p(y), _p(ys), _p(s))
+    return (y, ys, s) if want_s else (y, ys)
+
+
+def grouped_matmul_dequant(x, w, scale, per_token, group_list, list_type=0, w_trans=False, scale_dtype=DT_F32,
+                           out_dtype=DT_BF16, rows=None):
+    """Returns the output as fp32 (out_dtype 0) or raw uint16 bits (fp16 / bf16), shape [cnt, N]."""
+    x, w, M, K, N, gl, rows_a, cnt = _gemm_common(x, w, w_trans, group_list, rows)
+    sc = _c(scale, np.float32 if scale_dtype == DT_F32 else np.uint16)
+    pt = _c(per_token, np.float32)
+    out = np.zeros((cnt, N), np.float32 if out_dtype == DT_F32 else np.uint16)
+    lib().oracle_grouped_matmul_dequant(
+        _p(x), _p(w), ctypes.c_int(int(w_trans)), _p(sc), ctypes.c_int(scale_dtype), _p(pt), ctypes.c_int64(M),
+        ctypes.c_int64(K), ctypes.c_int64(N), ctypes.c_int64(gl.shape[0]), _p(gl), ctypes.c_int64(list_type), _p(rows_a),
+        ctypes.c_int64(cnt), _p(out), ctypes.c_int(out_dtype))
+    return out
+
+
+# ----------------------------------------------------------------------------------------------- finalize
+def moe_finalize_routing_v2(expanded_x, expanded_row_idx, x1=None, x2=None, bias=None, scales=None, expert_idx=None,
+                            drop_pad_mode=0, dtype=DT_F32, scale_dtype=None):
+    """expanded_x/x1/x2/bias: fp32 arrays (dtype 0) or uint16 bit arrays (dtype 1/27); returns the same representation."""
+    np_t = np.float32 if dtype == DT_F32 else np.uint16
+    if scale_dtype is None:
+        scale_dtype = dtype
+    np_s = np.float32 if scale_dtype == DT_F32 else np.uint16
+    ex = _c(expanded_x, np_t)
+    H = ex.shape[-1]
+    idx = _c(expanded_row_idx, np.int32)
+    sc = _c(scales, np_s)
+    K = 1 if sc is None else sc.shape[1]
+    T = idx.shape[0] // K
+    out = np.zeros((T, H), np_t)
+    lib().oracle_moe_finalize_routing_v2(
+        _p(ex), _p(idx), _p(_c(x1, np_t)), _p(_c(x2, np_t)), _p(_c(bias, np_t)), _p(sc), _p(_c(expert_idx, np.int32)),
+        ctypes.c_int64(drop_pad_mode), ctypes.c_int64(T), ctypes.c_int64(K), ctypes.c_int64(H), ctypes.c_int(dtype),
+        ctypes.c_int(scale_dtype), _p(out))
+    return out

@@ -1,0 +1,140 @@
+"""Pins the finalize oracle: numpy closed form in fp32, the reference example literal
+(moe/moe_finalize_routing_v2/examples/test_aclnn_moe_finalize_routing_v2.cpp:102-110), arrangement equivalence and the
+shapes of the reference's seeded generator (moe/moe_finalize_routing_v2/tests/ut/op_kernel/test_moe_finalize_routing_v2.cpp,
+finalize_routing_v2_data/gen_data.py: np.random.seed(5), (E, H, K, BS) tuples)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import bf16_round
+
+
+def _closed_form_f32(ex, idx, x1, x2, bias, scales, expert_idx, mode):
+    """fp32 data: acc = x1 + x2; acc += (ex[d] + bias[e]) * s in ascending k; separate multiply and add."""
+    T, K = scales.shape
+    acc = np.zeros((T, ex.shape[-1]), np.float32)
+    if x1 is not None:
+        acc = acc + x1
+    if x2 is not None:
+        acc = acc + x2
+    ex2 = ex.reshape(-1, ex.shape[-1])
+    for k in range(K):
+        d = idx.reshape(T, K)[:, k] if mode >= 2 else idx.reshape(K, T)[k]
+        v = ex2[np.maximum(d, 0)]
+        if bias is not None:
+            v = v + bias[expert_idx[:, k]]
+        term = (v * scales[:, k:k + 1]).astype(np.float32)
+        if mode in (1, 3):
+            term = np.where((d == -1)[:, None], np.float32(0), term)
+        acc = (acc + term).astype(np.float32)
+    return acc
+
+
+# (E, H, K, BS) tuples of the reference's generator
+REF_SHAPES = [(3, 7, 2, 12), (10, 30, 2, 1024), (10, 30, 3, 10), (10, 30, 4, 10), (300, 7, 257, 12), (471, 30, 4, 933),
+              (702, 30, 5, 340), (592, 30, 6, 105), (16, 20, 4, 12)]
+
+
+@pytest.mark.parametrize("E,H,K,BS", REF_SHAPES)
+@pytest.mark.parametrize("mode", [0, 2])
+def test_fp32_matches_closed_form(oracle, E, H, K, BS, mode):
+    rng = np.random.default_rng(5)
+    ex = rng.standard_normal((BS * K, H)).astype(np.float32)
+    x1 = rng.standard_normal((BS, H)).astype(np.float32)
+    x2 = rng.standard_normal((BS, H)).astype(np.float32)
+    bias = rng.standard_normal((E, H)).astype(np.float32)
+    scales = rng.standard_normal((BS, K)).astype(np.float32)
+    expert_idx = rng.integers(0, E, (BS, K)).astype(np.int32)
+    idx = rng.permutation(BS * K).astype(np.int32)
+    ref = _closed_form_f32(ex, idx, x1, x2, bias, scales, expert_idx, mode)
+    got = oracle.moe_finalize_routing_v2(ex, idx, x1, x2, bias, scales, expert_idx, drop_pad_mode=mode)
+    assert np.array_equal(got, ref)
+
+
+def test_reference_example_literal(oracle):
+    ex = np.array([0.1, 1.1, 2.1, 3.1, 4.1, 5.1, 6.1, 7.1, 8.1, 9.1, 10.1, 11.1,
+                   0.1, 1.1, 2.1, 3.1, 4.1, 5.1, 6.1, 7.1, 8.1, 9.1, 10.1, 11.1], np.float32).reshape(6, 4)
+    x1 = np.array([0.2, 1.2, 2.2, 3.2, 4.2, 5.2, 6.2, 7.2, 8.2, 9.2, 10.2, 11.2], np.float32).reshape(3, 4)
+    bias = np.array([0.2, 0.4, 0.2, 0.4, 0.2, 0.4, 0.2, 0.4], np.float32).reshape(2, 4)
+    scales = np.array([1.3, 1.6, 1.2, 1.8, 1.2, 2.3], np.float32).reshape(3, 2)
+    expert_idx = np.array([0, 1, 0, 1, 0, 1], np.int32).reshape(3, 2)
+    row_idx = np.array([2, 1, 4, 3, 0, 5], np.int32)
+    got = oracle.moe_finalize_routing_v2(ex, row_idx, x1, x1, bias, scales, expert_idx, drop_pad_mode=0)
+    # hand evaluation of token 0, column 0: x1+x2 = 0.4; k=0: idx[0*3+0]=2 -> ex[2,0]=8.1 (+0.2)*1.3; k=1: idx[1*3+0]=3 -> ex[3,0]=0.1 (+0.2)*1.6
+    want00 = np.float32(np.float32(0.2) + np.float32(0.2))
+    want00 = np.float32(want00 + np.float32(np.float32(np.float32(8.1) + np.float32(0.2)) * np.float32(1.3)))
+    want00 = np.float32(want00 + np.float32(np.float32(np.float32(0.1) + np.float32(0.2)) * np.float32(1.6)))
+    assert got[0, 0] == want00
+    assert np.array_equal(got, _closed_form_f32(ex, row_idx, x1, x1, bias, scales, expert_idx, 0))
+
+
+def test_row_and_column_arrangements_agree(oracle):
+    rng = np.random.default_rng(8)
+    T, K, H = 33, 4, 16
+    ex = rng.standard_normal((T * K, H)).astype(np.float32)
+    scales = rng.standard_normal((T, K)).astype(np.float32)
+    idx_row = rng.permutation(T * K).astype(np.int32)              # [n*K + k]
+    idx_col = np.ascontiguousarray(idx_row.reshape(T, K).T).reshape(-1)  # [k*T + n]
+    a = oracle.moe_finalize_routing_v2(ex, idx_row, scales=scales, drop_pad_mode=2)
+    b = oracle.moe_finalize_routing_v2(ex, idx_col, scales=scales, drop_pad_mode=0)
+    assert np.array_equal(a, b)
+
+
+def test_no_scales_is_plain_gather(oracle):
+    rng = np.random.default_rng(9)
+    ex = rng.standard_normal((20, 8)).astype(np.float32)
+    idx = rng.permutation(20).astype(np.int32)
+    got = oracle.moe_finalize_routing_v2(ex, idx, drop_pad_mode=0)
+    assert np.array_equal(got, ex[idx])
+
+
+def test_dropped_rows_contribute_nothing(oracle):
+    rng = np.random.default_rng(10)
+    T, K, H, E, C = 12, 3, 8, 4, 5
+    ex = rng.standard_normal((E, C, H)).astype(np.float32)
+    scales = rng.standard_normal((T, K)).astype(np.float32)
+    idx = rng.integers(-1, E * C, T * K).astype(np.int32)
+    idx[:K] = -1  # a token whose every row was dropped -> zeros
+    ref = _closed_form_f32(ex, idx, None, None, None, scales, None, 3)
+    got = oracle.moe_finalize_routing_v2(ex, idx, scales=scales, drop_pad_mode=3)
+    assert np.array_equal(got, ref)
+    assert (got[0] == 0).all()
+
+
+@pytest.mark.parametrize("scale_f32", [True, False])
+def test_bf16_accumulates_in_fp32_and_rounds_once(oracle, scale_f32):
+    rng = np.random.default_rng(12)
+    T, K, H, E = 40, 8, 64, 6
+    ex = bf16_round(rng.standard_normal((T * K, H)))
+    x1 = bf16_round(rng.standard_normal((T, H)))
+    bias = bf16_round(rng.standard_normal((E, H)))
+    scales = rng.uniform(0, 1, (T, K)).astype(np.float32)
+    if not scale_f32:
+        scales = bf16_round(scales)
+    expert_idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    idx = rng.permutation(T * K).astype(np.int32)
+    ref32 = _closed_form_f32(ex, idx, x1, None, bias, scales, expert_idx, 2)
+    ref = torch.from_numpy(ref32).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    b = oracle.f32_to_bf16_bits
+    got = oracle.moe_finalize_routing_v2(b(ex), idx, b(x1), None, b(bias), scales if scale_f32 else b(scales), expert_idx,
+                                         drop_pad_mode=2, dtype=oracle.DT_BF16,
+                                         scale_dtype=oracle.DT_F32 if scale_f32 else oracle.DT_BF16)
+    assert np.array_equal(got, ref)
+
+
+def test_fp16_rounds_after_every_operation(oracle):
+    rng = np.random.default_rng(13)
+    T, K, H = 25, 4, 32
+    h = np.float16
+    ex = rng.standard_normal((T * K, H)).astype(h)
+    x1 = rng.standard_normal((T, H)).astype(h)
+    x2 = rng.standard_normal((T, H)).astype(h)
+    scales = rng.uniform(0, 1, (T, K)).astype(h)
+    idx = rng.permutation(T * K).astype(np.int32)
+    acc = (x1 + x2).astype(h)  # numpy float16 arithmetic rounds every operation
+    for k in range(K):
+        term = (ex[idx.reshape(T, K)[:, k]] * scales[:, k:k + 1]).astype(h)
+        acc = (acc + term).astype(h)
+    got = oracle.moe_finalize_routing_v2(ex.view(np.uint16), idx, x1.view(np.uint16), x2.view(np.uint16), None,
+                                         scales.view(np.uint16), None, drop_pad_mode=2, dtype=oracle.DT_F16)
+    assert np.array_equal(got, acc.view(np.uint16))

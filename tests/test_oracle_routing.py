@@ -1,0 +1,105 @@
+"""Pins the routing oracle: numpy stable argsort / bincount (what every golden script of the reference uses,
+moe/moe_init_routing_quant_v2/tests/ut/op_kernel/moe_init_routing_quant_v2_data/gen_data.py:38-39), a brute-force
+restatement of drop/pad, invariants, and the literal of the reference example
+(moe/moe_init_routing_v2/examples/test_aclnn_moe_init_routing_v2.cpp:71-96)."""
+import numpy as np
+import pytest
+
+
+def _numpy_dropless(x, idx, E, active_num=0):
+    T, K = idx.shape
+    flat = idx.reshape(-1)
+    order = np.argsort(flat, kind="stable")
+    row_idx = np.empty(T * K, np.int32)
+    row_idx[order] = np.arange(T * K, dtype=np.int32)
+    hist = np.bincount(flat, minlength=E)[:E].astype(np.int32)
+    rows = T * K if active_num == 0 else min(T * K, active_num)
+    expanded = x[order[:rows] // K]
+    return expanded, row_idx, hist
+
+
+def _brute_drop_pad(x, idx, E, C):
+    T, K = idx.shape
+    flat = idx.reshape(-1)
+    row_idx = np.full(T * K, -1, np.int32)
+    expanded = np.zeros((E, C, x.shape[1]), x.dtype)
+    seen = [0] * E
+    for i in range(T * K):  # ascending flat index == stable rank within the expert
+        e = flat[i]
+        if seen[e] < C:
+            row_idx[i] = e * C + seen[e]
+            expanded[e, seen[e]] = x[i // K]
+        seen[e] += 1
+    return expanded, row_idx, np.array(seen, np.int32)
+
+
+@pytest.mark.parametrize("T,K,E,H", [(1, 1, 1, 1), (7, 3, 5, 4), (64, 8, 256, 16), (333, 2, 8, 7), (1000, 4, 33, 3)])
+def test_dropless_matches_numpy(oracle, T, K, E, H):
+    rng = np.random.default_rng(T * 131 + K)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    ex_ref, ri_ref, hist = _numpy_dropless(x, idx, E)
+    for flag in (0, 1, 2):
+        ex, ri, cnt, bef = oracle.moe_init_routing_v2(x, idx, expert_num=E, count_flag=flag)
+        assert np.array_equal(ri, ri_ref)
+        assert np.array_equal(ex, ex_ref)
+        assert bef is None
+        if flag == 0:
+            assert cnt is None
+        elif flag == 1:
+            assert np.array_equal(cnt, np.cumsum(hist).astype(np.int32))
+            assert cnt[-1] == T * K
+        else:
+            assert np.array_equal(cnt, hist)
+    # invariants: permutation, sortedness of the gathered expert ids, gather identity
+    assert np.array_equal(np.sort(ri_ref), np.arange(T * K))
+    sorted_e = np.empty(T * K, np.int32)
+    sorted_e[ri_ref] = idx.reshape(-1)
+    assert (np.diff(sorted_e) >= 0).all()
+
+
+def test_active_num_truncates_rows(oracle):
+    rng = np.random.default_rng(5)
+    T, K, E, H = 50, 4, 9, 6
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    for active in (1, 37, 199, 200, 5000):
+        ex_ref, ri_ref, _ = _numpy_dropless(x, idx, E, active)
+        ex, ri, _, _ = oracle.moe_init_routing_v2(x, idx, active_num=active, expert_num=E)
+        assert ex.shape == ex_ref.shape
+        assert np.array_equal(ex, ex_ref) and np.array_equal(ri, ri_ref)
+
+
+@pytest.mark.parametrize("T,K,E,C", [(3, 2, 3, 2), (40, 4, 6, 5), (40, 4, 6, 40), (128, 8, 16, 3)])
+def test_drop_pad_matches_brute_force(oracle, T, K, E, C):
+    rng = np.random.default_rng(T + C)
+    x = rng.standard_normal((T, 5)).astype(np.float32)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    ex_ref, ri_ref, hist = _brute_drop_pad(x, idx, E, C)
+    ex, ri, cnt, bef = oracle.moe_init_routing_v2(x, idx, expert_capacity=C, expert_num=E, drop_pad_mode=1,
+                                                  count_flag=1, before_capacity_flag=True)
+    assert cnt is None  # drop/pad never emits count-or-cumsum
+    assert np.array_equal(ri, ri_ref) and np.array_equal(ex, ex_ref) and np.array_equal(bef, hist)
+
+
+def test_reference_example_literal(oracle):
+    # x rows 0.1 / 0.2 / 0.3, expertIdx {1,2,0,1,0,2}, E=3, C=2, drop/pad, before-capacity counts requested
+    x = np.repeat(np.array([[0.1], [0.2], [0.3]], np.float32), 4, axis=1)
+    idx = np.array([[1, 2], [0, 1], [0, 2]], np.int32)
+    ex, ri, cnt, bef = oracle.moe_init_routing_v2(x, idx, expert_capacity=2, expert_num=3, drop_pad_mode=1,
+                                                  before_capacity_flag=True)
+    assert ri.tolist() == [2, 4, 0, 3, 1, 5]
+    assert bef.tolist() == [2, 2, 2]
+    want = np.array([[0.2, 0.3], [0.1, 0.2], [0.1, 0.3]], np.float32)  # token rows per expert slot
+    assert np.array_equal(ex[:, :, 0], want)
+
+
+def test_unknown_expert_range_sorts_signed(oracle):
+    rng = np.random.default_rng(11)
+    idx = rng.integers(-50, 5000, (200, 3)).astype(np.int32)
+    x = rng.standard_normal((200, 2)).astype(np.float32)
+    ex, ri, _, _ = oracle.moe_init_routing_v2(x, idx, expert_num=0)
+    order = np.argsort(idx.reshape(-1), kind="stable")
+    ref = np.empty(600, np.int32)
+    ref[order] = np.arange(600, dtype=np.int32)
+    assert np.array_equal(ri, ref)
