@@ -1,0 +1,161 @@
+"""The grouped int8 GEMM operators on the GPU against the CPU oracle.
+
+Bars: int32 accumulators bit-exact; bf16 / fp16 outputs of the down projection bit-exact (same fp32 operation order,
+nearest-even casts); SwiGLU-quant int8 within +-1 LSB and scales within 1e-2 relative (in practice ~1e-6: only the
+device's expf and divide can differ from the host's).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(rng, M, K, N, E, mode="ragged"):
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)  # K-contiguous storage
+    if mode == "ragged":
+        cuts = np.sort(rng.integers(0, M + 1, E - 1)) if E > 1 else np.array([], np.int64)
+        cumsum = np.concatenate([cuts, [M]]).astype(np.int64)
+    elif mode == "even":
+        cumsum = ((np.arange(1, E + 1) * M) // E).astype(np.int64)
+    elif mode == "sparse":  # most groups empty
+        sizes = np.zeros(E, np.int64)
+        hot = rng.choice(E, max(1, E // 8), replace=False)
+        sizes[hot] = rng.multinomial(M, np.ones(len(hot)) / len(hot))
+        cumsum = np.cumsum(sizes)
+    return x, wt, cumsum
+
+
+def _weight_views(wt, dev, layout):
+    """[E, K, N] view for the operator: transposed view of K-contiguous storage, or a contiguous ND tensor."""
+    w_dev = torch.from_numpy(wt).to(dev)
+    if layout == "kmajor":
+        return w_dev.transpose(1, 2)
+    return w_dev.transpose(1, 2).contiguous()
+
+
+INT32_CASES = [  # M, K, N, E, mode, layout
+    (1, 16, 8, 1, "even", "kmajor"),
+    (37, 128, 24, 4, "ragged", "kmajor"),
+    (96, 256, 300, 7, "ragged", "kmajor"),
+    (512, 1024, 512, 8, "even", "kmajor"),       # tile 96
+    (512, 4096, 256, 128, "ragged", "kmajor"),   # decode-like: tile 32, many groups
+    (700, 512, 520, 3, "ragged", "kmajor"),      # tile 256, N not a multiple of the tile
+    (1500, 384, 256, 10, "ragged", "kmajor"),    # tile 192 + partial tiles
+    (2048, 2048, 256, 16, "even", "kmajor"),     # tile 192, exact 128-row groups
+    (300, 200, 64, 4, "ragged", "kmajor"),       # K not a multiple of 16: byte-wise loader
+    (300, 208, 72, 4, "ragged", "nd"),           # row-major [E,K,N] weight: byte-wise loader
+    (100, 7168, 64, 2, "even", "kmajor"),        # |acc| beyond 2^24
+    (640, 256, 256, 64, "sparse", "kmajor"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,E,mode,layout", INT32_CASES)
+def test_int32_accumulators_bit_exact(aclnn, oracle, dev, M, K, N, E, mode, layout):
+    rng = np.random.default_rng(M * 3 + K + N)
+    x, wt, cumsum = _problem(rng, M, K, N, E, mode)
+    ref = oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)
+    xd = torch.from_numpy(x).to(dev)
+    wv = _weight_views(wt, dev, layout)
+    for list_type, dtype in ((0, torch.int64), (1, torch.int64), (0, torch.int32)):
+        gl = cumsum if list_type == 0 else np.diff(np.concatenate([[0], cumsum]))
+        out = torch.full((M, N), -7, dtype=torch.int32, device=dev)
+        aclnn.grouped_matmul_v4([xd], [wv], group_list=torch.from_numpy(gl).to(dev).to(dtype), split_item=3, group_type=0,
+                                group_list_type=list_type, out=[out])
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), ref)
+
+
+def test_rows_beyond_last_group_untouched(aclnn, oracle, dev):
+    rng = np.random.default_rng(4)
+    x, wt, _ = _problem(rng, 200, 128, 64, 3, "even")
+    cumsum = np.array([50, 50, 120], np.int64)
+    out = torch.full((200, 64), -7, dtype=torch.int32, device=dev)
+    aclnn.grouped_matmul_v4([torch.from_numpy(x).to(dev)], [_weight_views(wt, dev, "kmajor")],
+                            group_list=torch.from_numpy(cumsum).to(dev), split_item=3, group_type=0, out=[out])
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    ref = oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)
+    assert np.array_equal(got[:120], ref[:120]) and (got[120:] == -7).all()
+
+
+DEQUANT_CASES = [(64, 256, 128, 4, "f32", torch.bfloat16), (64, 256, 128, 4, "bf16", torch.bfloat16),
+                 (64, 256, 128, 4, "f32", torch.float16), (512, 1024, 1024, 8, "f32", torch.bfloat16),
+                 (333, 1536, 520, 16, "f32", torch.bfloat16)]
+
+
+@pytest.mark.parametrize("M,K,N,E,scale_dtype,out_dtype", DEQUANT_CASES)
+def test_down_projection_epilogue(aclnn, oracle, dev, M, K, N, E, scale_dtype, out_dtype):
+    rng = np.random.default_rng(M + N)
+    x, wt, cumsum = _problem(rng, M, K, N, E)
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    per_token = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    scale_t = torch.from_numpy(scale).to(dev)
+    if scale_dtype == "bf16":
+        scale_t = scale_t.to(torch.bfloat16)
+        scale_arg, sd = scale_t.view(torch.int16).cpu().numpy().view(np.uint16), oracle.DT_BF16
+    else:
+        scale_arg, sd = scale, oracle.DT_F32
+    od = oracle.DT_BF16 if out_dtype == torch.bfloat16 else oracle.DT_F16
+    ref = oracle.grouped_matmul_dequant(x, wt, scale_arg, per_token, cumsum, w_trans=True, scale_dtype=sd, out_dtype=od)
+    out = aclnn.grouped_matmul_v4([torch.from_numpy(x).to(dev)], [_weight_views(wt, dev, "kmajor")], scale=[scale_t],
+                                  per_token_scale=[torch.from_numpy(per_token).to(dev)],
+                                  group_list=torch.from_numpy(cumsum).to(dev), split_item=3, group_type=0,
+                                  output_dtype=out_dtype)[0]
+    torch.cuda.synchronize()
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+
+
+SWIGLU_CASES = [  # M, K, N, E, mode, layout, scale dtype
+    (16, 256, 512, 4, "even", "kmajor", "f32"),       # reference tiling UT shape
+    (192, 2048, 2048, 4, "ragged", "kmajor", "f32"),  # reference op_api UT shape
+    (512, 1024, 2048, 8, "ragged", "kmajor", "f32"),  # small config
+    (512, 4096, 3072, 128, "ragged", "kmajor", "f32"),  # decode config shape
+    (300, 512, 208, 5, "ragged", "kmajor", "bf16"),   # N/2 not a multiple of the tile
+    (300, 512, 208, 5, "ragged", "kmajor", "f16"),
+    (100, 200, 96, 3, "ragged", "nd", "f32"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,E,mode,layout,sdt", SWIGLU_CASES)
+def test_swiglu_quant(aclnn, oracle, dev, M, K, N, E, mode, layout, sdt):
+    rng = np.random.default_rng(M + K + N)
+    x, wt, cumsum = _problem(rng, M, K, N, E, mode)
+    used = int(M * 0.9)
+    cumsum = np.minimum(cumsum, used)  # trailing rows belong to no group and must stay untouched
+    w_scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    x_scale = rng.uniform(5e-3, 5e-2, M).astype(np.float32)
+    ws_t = torch.from_numpy(w_scale).to(dev)
+    if sdt == "bf16":
+        ws_t = ws_t.to(torch.bfloat16)
+        ws_arg, code = ws_t.view(torch.int16).cpu().numpy().view(np.uint16), oracle.DT_BF16
+    elif sdt == "f16":
+        ws_t = ws_t.to(torch.float16)
+        ws_arg, code = ws_t.view(torch.int16).cpu().numpy().view(np.uint16), oracle.DT_F16
+    else:
+        ws_arg, code = w_scale, oracle.DT_F32
+    y_ref, ys_ref = oracle.grouped_matmul_swiglu_quant(x, wt, ws_arg, x_scale, cumsum, w_trans=True, w_scale_dtype=code)
+    y = torch.full((M, N // 2), 55, dtype=torch.int8, device=dev)
+    ys = torch.full((M,), -3.0, dtype=torch.float32, device=dev)
+    aclnn.grouped_matmul_swiglu_quant(torch.from_numpy(x).to(dev), _weight_views(wt, dev, layout),
+                                      torch.from_numpy(cumsum).to(dev), ws_t, torch.from_numpy(x_scale).to(dev),
+                                      out=(y, ys))
+    torch.cuda.synchronize()
+    y, ys = y.cpu().numpy(), ys.cpu().numpy()
+    last = int(cumsum[-1])
+    diff = np.abs(y[:last].astype(np.int32) - y_ref[:last].astype(np.int32))
+    assert diff.max() <= 1, "int8 output differs by %d LSB" % diff.max()
+    assert (diff != 0).mean() < 1e-3
+    np.testing.assert_allclose(ys[:last], ys_ref[:last], rtol=1e-2)
+    np.testing.assert_allclose(ys[:last], ys_ref[:last], rtol=1e-5)  # observed: only expf / divide rounding differs
+    assert (y[last:] == 55).all() and (ys[last:] == -3.0).all()
+
+
+def test_swiglu_empty_group_list_is_noop(aclnn, dev):
+    x = torch.zeros((4, 32), dtype=torch.int8, device=dev)
+    w = torch.zeros((2, 64, 32), dtype=torch.int8, device=dev).transpose(1, 2)
+    gl = torch.empty((0,), dtype=torch.int64, device=dev)
+    y, ys = aclnn.grouped_matmul_swiglu_quant(x, w, gl, torch.ones((2, 64), device=dev), torch.ones((4,), device=dev))
+    torch.cuda.synchronize()
+    assert y.shape == (4, 32)

@@ -1,0 +1,119 @@
+"""aclnnMoeInitRoutingV2 on the GPU against the CPU oracle: bit-exact indices, counts and gathered rows."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(aclnn, dev, x, idx, **kw):
+    outs = aclnn.moe_init_routing_v2(torch.from_numpy(x).to(dev), torch.from_numpy(idx).to(dev), **kw)
+    torch.cuda.synchronize()
+    return [None if o is None else o.cpu().numpy() for o in outs]
+
+
+CASES = [  # T, K, E, H, dtype
+    (1, 1, 1, 1, np.float32),
+    (3, 2, 3, 4, np.float32),
+    (7, 3, 5, 30, np.float16),
+    (64, 8, 128, 4096, np.int8),       # decode shape
+    (256, 2, 8, 1024, np.int8),        # small config
+    (333, 5, 100, 7, np.float32),      # odd row bytes
+    (1000, 4, 33, 18, np.int8),        # 18-byte rows: 2-byte vector path
+    (4096, 8, 256, 512, np.float16),   # DeepSeek-V3 routing shape (narrow rows keep the host copy small)
+    (2048, 6, 2000, 8, np.float32),    # 11-bit digit
+]
+
+
+@pytest.mark.parametrize("T,K,E,H,dtype", CASES)
+def test_dropless_bit_exact(aclnn, oracle, dev, T, K, E, H, dtype):
+    rng = np.random.default_rng(T * 7 + K)
+    x = (rng.standard_normal((T, H)) * 50).astype(dtype)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    for flag in (1, 2, 0):
+        ex, ri, cnt, _ = _run(aclnn, dev, x, idx, expert_num=E, expert_tokens_count_or_cumsum_flag=flag)
+        ex_r, ri_r, cnt_r, _ = oracle.moe_init_routing_v2(x, idx, expert_num=E, count_flag=flag)
+        assert np.array_equal(ri, ri_r)
+        assert np.array_equal(ex.view(np.uint8), ex_r.view(np.uint8))
+        if flag:
+            assert np.array_equal(cnt, cnt_r)
+        else:
+            assert cnt is None
+
+
+def test_skewed_routing_bit_exact(pkg, aclnn, oracle, dev):
+    """Zipf-skewed load on the DeepSeek-V3 expert count: many empty experts, one very hot expert."""
+    cfg = pkg.synth.config(4)
+    idx, _ = pkg.synth.make_routing(cfg, seed=4)
+    hist = np.bincount(idx.reshape(-1), minlength=cfg.experts)
+    assert (hist == 0).mean() > 0.2 and hist.max() > 10 * hist.mean()
+    x = np.arange(cfg.tokens * 16, dtype=np.int32).reshape(cfg.tokens, 16).view(np.float32)
+    for flag in (1, 2):
+        ex, ri, cnt, _ = _run(aclnn, dev, x, idx, expert_num=cfg.experts, expert_tokens_count_or_cumsum_flag=flag)
+        ex_r, ri_r, cnt_r, _ = oracle.moe_init_routing_v2(x, idx, expert_num=cfg.experts, count_flag=flag)
+        assert np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r)
+        assert np.array_equal(ex.view(np.uint32), ex_r.view(np.uint32))
+
+
+def test_active_num(aclnn, oracle, dev):
+    rng = np.random.default_rng(3)
+    T, K, E, H = 100, 4, 16, 32
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    for active in (1, 123, 400, 9999):
+        ex, ri, _, _ = _run(aclnn, dev, x, idx, active_num=active, expert_num=E)
+        ex_r, ri_r, _, _ = oracle.moe_init_routing_v2(x, idx, active_num=active, expert_num=E)
+        assert ex.shape == ex_r.shape and np.array_equal(ex, ex_r) and np.array_equal(ri, ri_r)
+
+
+@pytest.mark.parametrize("T,K,E,C,H", [(3, 2, 3, 2, 4), (128, 8, 16, 3, 64), (500, 4, 7, 400, 10), (64, 2, 40, 1, 8)])
+def test_drop_pad_bit_exact(aclnn, oracle, dev, T, K, E, C, H):
+    rng = np.random.default_rng(T + C)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    ex, ri, cnt, bef = _run(aclnn, dev, x, idx, expert_capacity=C, expert_num=E, drop_pad_mode=1,
+                            expert_tokens_count_or_cumsum_flag=1, expert_tokens_before_capacity_flag=True)
+    ex_r, ri_r, _, bef_r = oracle.moe_init_routing_v2(x, idx, expert_capacity=C, expert_num=E, drop_pad_mode=1,
+                                                      count_flag=1, before_capacity_flag=True)
+    assert cnt is None
+    assert np.array_equal(ri, ri_r) and np.array_equal(bef, bef_r) and np.array_equal(ex, ex_r)
+
+
+def test_reference_example(aclnn, dev):
+    """Literal of moe/moe_init_routing_v2/examples/test_aclnn_moe_init_routing_v2.cpp:71-96."""
+    x = np.repeat(np.array([[0.1], [0.2], [0.3]], np.float32), 4, axis=1)
+    idx = np.array([[1, 2], [0, 1], [0, 2]], np.int32)
+    ex, ri, _, bef = _run(aclnn, dev, x, idx, expert_capacity=2, expert_num=3, drop_pad_mode=1,
+                          expert_tokens_before_capacity_flag=True)
+    assert ri.tolist() == [2, 4, 0, 3, 1, 5] and bef.tolist() == [2, 2, 2]
+    assert np.array_equal(ex[:, :, 0], np.array([[0.2, 0.3], [0.1, 0.2], [0.1, 0.3]], np.float32))
+
+
+def test_unknown_expert_range(aclnn, oracle, dev):
+    """expertNum 0: the id range is unknown, ids sort as signed 32-bit integers (three digit passes)."""
+    rng = np.random.default_rng(11)
+    idx = rng.integers(-50, 5000, (700, 3)).astype(np.int32)
+    x = rng.standard_normal((700, 6)).astype(np.float32)
+    ex, ri, _, _ = _run(aclnn, dev, x, idx, expert_num=0)
+    ex_r, ri_r, _, _ = oracle.moe_init_routing_v2(x, idx, expert_num=0)
+    assert np.array_equal(ri, ri_r) and np.array_equal(ex, ex_r)
+
+
+def test_many_experts_counts(aclnn, oracle, dev):
+    """More than 2048 experts: two digit passes, counts from the sorted keys."""
+    rng = np.random.default_rng(12)
+    E = 5000
+    idx = rng.integers(0, E, (3000, 2)).astype(np.int32)
+    x = rng.standard_normal((3000, 4)).astype(np.float32)
+    for flag in (1, 2):
+        ex, ri, cnt, _ = _run(aclnn, dev, x, idx, expert_num=E, expert_tokens_count_or_cumsum_flag=flag)
+        ex_r, ri_r, cnt_r, _ = oracle.moe_init_routing_v2(x, idx, expert_num=E, count_flag=flag)
+        assert np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r) and np.array_equal(ex, ex_r)
+
+
+def test_empty_inputs(aclnn, dev):
+    x = torch.empty((0, 16), dtype=torch.float32, device=dev)
+    idx = torch.empty((0, 4), dtype=torch.int32, device=dev)
+    ex, ri, _, _ = aclnn.moe_init_routing_v2(x, idx, expert_num=4)
+    torch.cuda.synchronize()
+    assert ex.shape == (0, 16) and ri.shape == (0,)
