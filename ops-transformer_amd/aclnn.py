@@ -301,3 +301,28 @@ def moe_finalize_routing_v2(expanded_x, expanded_row_idx, x1=None, x2=None, bias
     finally:
         h.close()
     return out
+
+
+# ------------------------------------------------------------------------------------------------ kernel timing
+def kernel_timer_enable(enable=True):
+    """Turns per-kernel HIP-event timing inside the library on or off (include/opapi_profile.h)."""
+    l = lib()
+    l.opapiKernelTimerEnable.argtypes = [ctypes.c_int]
+    l.opapiKernelTimerEnable.restype = None
+    l.opapiKernelTimerEnable(1 if enable else 0)
+
+
+def kernel_timer_report():
+    """Waits for the recorded launches and returns {kernel name: (launches, total milliseconds)}."""
+    l = lib()
+    l.opapiKernelTimerReport.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
+    l.opapiKernelTimerReport.restype = ctypes.c_int
+    buf = ctypes.create_string_buffer(1 << 14)
+    rc = l.opapiKernelTimerReport(buf, len(buf))
+    if rc < 0:
+        raise RuntimeError("opapiKernelTimerReport failed")
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, count, total = line.split()
+        out[name] = (int(count), float(total))
+    return out

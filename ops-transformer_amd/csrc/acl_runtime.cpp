@@ -4,7 +4,10 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <new>
+
+#include "opapi_profile.h"
 
 namespace {
 thread_local std::string g_lastError;
@@ -70,9 +73,70 @@ aclnnStatus RunAndRelease(void* workspace, uint64_t workspaceSize, aclOpExecutor
     return st;
 }
 
+namespace {
+struct TimedLaunch {
+    const char* name;
+    hipEvent_t start, stop;
+};
+bool g_timerOn = false;
+std::vector<TimedLaunch> g_timed;
+
+void DropTimed() {
+    for (TimedLaunch& t : g_timed) {
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+    }
+    g_timed.clear();
+}
+}  // namespace
+
+KernelTimer::KernelTimer(const char* name, hipStream_t stream) : name_(name), stream_(stream) {
+    if (!g_timerOn) return;
+    if (hipEventCreate(&start_) != hipSuccess) { start_ = nullptr; return; }
+    (void)hipEventRecord(start_, stream_);
+}
+
+KernelTimer::~KernelTimer() {
+    if (start_ == nullptr) return;
+    hipEvent_t stop = nullptr;
+    if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start_); return; }
+    (void)hipEventRecord(stop, stream_);
+    g_timed.push_back({name_, start_, stop});
+}
+
 }  // namespace opapi
 
 extern "C" {
+
+void opapiKernelTimerEnable(int enable) {
+    opapi::DropTimed();
+    opapi::g_timerOn = enable != 0;
+}
+
+int opapiKernelTimerReport(char* buf, size_t cap) {
+    std::map<std::string, std::pair<int, double>> agg;
+    int rc = 0;
+    for (opapi::TimedLaunch& t : opapi::g_timed) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(t.stop) != hipSuccess || hipEventElapsedTime(&ms, t.start, t.stop) != hipSuccess) rc = -1;
+        auto& a = agg[t.name];
+        a.first += 1;
+        a.second += ms;
+    }
+    opapi::DropTimed();
+    std::string out;
+    for (auto& kv : agg) {
+        char line[256];
+        snprintf(line, sizeof(line), "%s %d %.6f\n", kv.first.c_str(), kv.second.first, kv.second.second);
+        out += line;
+    }
+    if (buf != nullptr && cap > 0) {
+        const size_t n = out.size() < cap - 1 ? out.size() : cap - 1;
+        memcpy(buf, out.data(), n);
+        buf[n] = '\0';
+    }
+    return rc < 0 ? rc : static_cast<int>(agg.size());
+}
 
 aclError aclInit(const char*) { return ACL_SUCCESS; }
 aclError aclFinalize(void) { return ACL_SUCCESS; }

@@ -25,6 +25,8 @@
 // [K, N] form and shapes whose K is not a multiple of 16 go through a byte-wise loader that is correct but slow.
 #include "grouped_gemm_i8.h"
 
+#include "opapi_common.h"
+
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
@@ -536,7 +538,10 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     sa.isCount = p.groupListKind == GroupListKind::kCount ? 1 : 0;
     sa.tileM = plan.tileM;
     sa.M = p.M;
-    hipLaunchKernelGGL(ScheduleKernel, dim3(1), dim3(1024), 0, stream, sa);
+    {
+        opapi::KernelTimer timer("gmm_schedule", stream);
+        hipLaunchKernelGGL(ScheduleKernel, dim3(1), dim3(1024), 0, stream, sa);
+    }
 
     KernelArgs ka{};
     ka.x = p.x;
@@ -562,6 +567,8 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     hipError_t e = hipSuccess;
     if (p.K > 0) {
         const bool fast = FastLoadOk(p);
+        opapi::KernelTimer timer(p.epilogue == Epilogue::kSwiglu ? "gmm_swiglu"
+                                 : p.epilogue == Epilogue::kDequant ? "gmm_dequant" : "gmm_int32", stream);
         switch (p.epilogue) {
             case Epilogue::kInt32:
                 e = fast ? LaunchShape<Epilogue::kInt32, true>(plan, ka, plan.maxTiles, stream)
@@ -580,6 +587,7 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     }
     if (swiglu) {
         RequantArgs ra{sBuf, rowMax, sched, p.quantOut, p.quantScaleOut, static_cast<int32_t>(p.N / 2)};
+        opapi::KernelTimer timer("gmm_requant", stream);
         hipLaunchKernelGGL(RequantKernel, dim3(static_cast<unsigned>(p.M)), dim3(256), 0, stream, ra);
         e = hipGetLastError();
     }

@@ -163,6 +163,7 @@ class FinalizeExecutor : public aclOpExecutor {
 
     aclnnStatus Run(void*, hipStream_t stream) override {
         if (args.tokens == 0 || args.hidden == 0) return ACLNN_SUCCESS;
+        opapi::KernelTimer timer("finalize", stream);
         if (dtype == ACL_BF16) {
             if (vectorOk) Launch<Bf16Codec, 8>(stream); else Launch<Bf16Codec, 1>(stream);
         } else if (dtype == ACL_FLOAT16) {

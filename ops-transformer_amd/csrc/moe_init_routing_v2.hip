@@ -360,9 +360,18 @@ class InitRoutingExecutor : public aclOpExecutor {
                 co.beforeCapacity = beforeCapacity;
             }
             InverseMap im{last ? expandedRowIdx : nullptr, dropPad, static_cast<int32_t>(capacity)};
-            hipLaunchKernelGGL(DigitHistogramKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p);
-            hipLaunchKernelGGL(DigitScanKernel, dim3(1), dim3(1024), 0, stream, p, co);
-            hipLaunchKernelGGL(DigitScatterKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p, im);
+            {
+                opapi::KernelTimer timer("routing_histogram", stream);
+                hipLaunchKernelGGL(DigitHistogramKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p);
+            }
+            {
+                opapi::KernelTimer timer("routing_scan", stream);
+                hipLaunchKernelGGL(DigitScanKernel, dim3(1), dim3(1024), 0, stream, p, co);
+            }
+            {
+                opapi::KernelTimer timer("routing_scatter", stream);
+                hipLaunchKernelGGL(DigitScatterKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p, im);
+            }
             keysIn = p.keysOut;
             payloadIn = p.payloadOut;
             shift += bitsPerPass[pass];
@@ -373,6 +382,7 @@ class InitRoutingExecutor : public aclOpExecutor {
             hipLaunchKernelGGL(CountFromSortedKernel, dim3(blocks), dim3(256), 0, stream, keysIn, total, co);
         }
         if (rowBytes > 0 && tokens > 0) {
+            opapi::KernelTimer timer("routing_gather", stream);
             const uintptr_t align = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(expandedX) |
                                     static_cast<uintptr_t>(rowBytes);
             if (align % 16 == 0) LaunchGather<uint4>(ws, stream);

@@ -98,6 +98,21 @@ inline uint64_t AlignUp(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
 std::string ShapeStr(const aclTensor* t);
 
+// Brackets the kernel launches made during its lifetime with HIP events on `stream` when kernel timing is enabled
+// (include/opapi_profile.h); otherwise does nothing.
+class KernelTimer {
+   public:
+    KernelTimer(const char* name, hipStream_t stream);
+    ~KernelTimer();
+    KernelTimer(const KernelTimer&) = delete;
+    KernelTimer& operator=(const KernelTimer&) = delete;
+
+   private:
+    const char* name_;
+    hipStream_t stream_;
+    hipEvent_t start_ = nullptr;
+};
+
 }  // namespace opapi
 
 #define OPAPI_CHECK(cond, code, ...)            \
