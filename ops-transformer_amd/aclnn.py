@@ -12,7 +12,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "lib", "libcust_opapi.so")
+_LIB_PATH = os.environ.get("OPAPI_LIBRARY_PATH") or os.path.join(_HERE, "lib", "libcust_opapi.so")
 
 ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32, ACL_INT64, ACL_BF16 = 0, 1, 2, 3, 9, 27
 ACL_FORMAT_ND = 2

@@ -7,29 +7,30 @@
 //            (reference order: gmm/grouped_matmul/op_kernel/grouped_matmul_quant_mixcore.h:248-291,293-310)
 //   kSwiglu  C = (float(acc) * rowScale[r]) * scale[e, c];  S = swish(C[:, j]) * C[:, j + N/2]
 //            (reference order: gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:368-399,446-474),
-//            S is written as fp32 together with a per-row running max |S| (atomic max on the bit pattern); a second,
-//            bandwidth-trivial kernel turns S into int8 with the row scale max/127 (same file :477-513).
+//            S is written as fp32 together with one partial max |S| per (n-tile, row); a second, bandwidth-trivial
+//            kernel folds the partials and turns S into int8 with the row scale max/127 (same file :477-513).
 //
-// Structure.  Group sizes live in device memory, so a one-workgroup scheduling kernel turns groupList into
-// (row start, rows, m-tile prefix) per group; the GEMM grid is launched with a static upper bound of workgroups and
-// each workgroup finds its (group, m-tile, n-tile) by binary search, surplus workgroups exit at once.  Workgroup ids
-// are dealt round-robin to the 8 XCDs by the hardware, so logical tile index = xcd * ceil(total / 8) + id / 8 keeps
-// the tiles of one expert (which share activation rows and, across m-tiles, weight columns) on one XCD's L2.
+// Scheduling.  Group sizes live in device memory, so a one-workgroup kernel turns groupList into (row start, rows,
+// m-tile prefix) per group.  Tiles are ordered group-major and dealt to the 8 XCDs in contiguous shares, so the
+// workgroups of one XCD always sit on neighbouring tiles of the same expert (shared activation rows stay in that
+// XCD's L2); inside a group, bands of 4 m-tiles walk the n-tiles together so weight columns are reused from L2.
 //
-// Tile: (32 * subTilesM * wavesM) rows x 256 columns x 128 k-bytes per step; 4 wave columns, each owning two 32-wide
-// MFMA column tiles.  For kSwiglu the 256 columns are 128 "activated" columns j and their 128 partners j + N/2 and a
-// wave owns matching 32-column blocks of both, so the SwiGLU product is formed in registers.
-// Operands are staged global -> registers -> LDS with two LDS buffers; LDS rows are 128 bytes with the 16-byte chunk
-// index XOR-ed with (row & 7), which makes both the 16-byte stores and the MFMA operand loads bank-conflict free.
-// Weights are consumed K-contiguous ([N, K] per expert, the "transposed" view of the reference API); the row-major
-// [K, N] form and shapes whose K is not a multiple of 16 go through a byte-wise loader that is correct but slow.
+// Two kernels share the tile decode and the epilogue:
+//   StreamGemmKernel  the fast path (K-contiguous weights, K a multiple of 64).  Persistent workgroups; operands go
+//                     global -> LDS with global_load_lds_dwordx4 into a ring of 4..8 stages of 64 k-bytes, so several
+//                     stages of weights are in flight per CU with no staging registers, and the ring keeps filling
+//                     with the next tile's first steps while the current tile's epilogue runs.
+//   GenericGemmKernel byte-wise loader for row-major [K, N] weights and for K not a multiple of 64: correct, slow.
+// LDS rows are XOR-swizzled in 16-byte chunks so that the 16 lanes the LDS serves per clock (64 banks) never collide,
+// for the DMA writes as well as for the MFMA operand reads.
 #include "grouped_gemm_i8.h"
-
-#include "opapi_common.h"
 
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <type_traits>
+
+#include "opapi_common.h"
 
 namespace gemm {
 namespace {
@@ -37,14 +38,13 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kStepBytes = 128;  // k extent of one pipeline step (int8 elements == bytes)
 constexpr int kTileN = 256;
 constexpr int kWavesN = 4;
 constexpr int kChunk = 16;
-constexpr int kChunksPerRow = kStepBytes / kChunk;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // m-tiles walked together per n-tile for L2 reuse of weight columns
 constexpr int kMaxGroups = 1024;
+constexpr int kLdsBudget = 160 * 1024;
 
 // ---------------------------------------------------------------------------------------------- scheduling table
 // int32 layout: [0] total rows covered by groups, [1] total m-tiles, [2..2+G) row start, [..+G) rows, [..+G+1) m-tile prefix
@@ -53,7 +53,6 @@ __host__ __device__ inline int SchedInts(int groups) { return 2 + 3 * groups + 1
 struct SchedArgs {
     const void* groupList;
     int32_t* sched;
-    uint32_t* rowMax;  // zeroed for [0, M) when not null
     int32_t groups;
     int32_t groupListIsInt64;
     int32_t isCount;
@@ -116,12 +115,9 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
             a.sched[1] = tileInc;
         }
     }
-    if (a.rowMax != nullptr) {
-        for (int64_t i = t; i < a.M; i += 1024) a.rowMax[i] = 0u;
-    }
 }
 
-// ---------------------------------------------------------------------------------------------- GEMM kernel
+// ---------------------------------------------------------------------------------------------- shared device code
 struct KernelArgs {
     const int8_t* x;
     const int8_t* w;
@@ -139,10 +135,58 @@ struct KernelArgs {
     int32_t scaleDtype;
     const float* rowScale;
     float* sOut;
-    uint32_t* rowMax;
+    float* rowMax;  // [tilesN][M] partial max |S| per n-tile
 };
 
-__device__ __forceinline__ int LdsOffset(int row, int chunk) { return row * kStepBytes + ((chunk ^ (row & 7)) << 4); }
+// One output tile of one group, decoded from the scheduling table (all fields are wave-uniform).
+struct TileInfo {
+    int32_t valid;
+    int32_t group;
+    int32_t rowBase;  // first row of the tile in x / out
+    int32_t rows;     // 1..tileM real rows
+    int32_t tileN;
+    int32_t colBase;  // first output channel (kSwiglu: first column of S)
+};
+
+// Position `local` of the XCD share that starts at logical tile `xcdFirst`.
+template <int kTileM, bool kSwiglu>
+__device__ __forceinline__ TileInfo DecodeTile(const KernelArgs& a, int64_t xcdFirst, int64_t perXcd, int64_t totalTiles,
+                                               int64_t local) {
+    TileInfo t{};
+    const int64_t logical = xcdFirst + local;
+    if (local >= perXcd || logical >= totalTiles) return t;
+    const int32_t* const rowStartTbl = a.sched + 2;
+    const int32_t* const rowCountTbl = rowStartTbl + a.groups;
+    const int32_t* const tilePrefix = rowCountTbl + a.groups;
+    const int32_t q = static_cast<int32_t>(logical / a.tilesN);
+    int lo = 0, hi = a.groups;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tilePrefix[mid] <= q) lo = mid; else hi = mid;
+    }
+    const int32_t inGroup = static_cast<int32_t>(logical - static_cast<int64_t>(tilePrefix[lo]) * a.tilesN);
+    const int32_t tilesM = tilePrefix[lo + 1] - tilePrefix[lo];
+    const int32_t band = inGroup / (kGroupM * a.tilesN);
+    const int32_t rem = inGroup % (kGroupM * a.tilesN);
+    const int32_t bandTiles = min(kGroupM, tilesM - kGroupM * band);
+    const int32_t tileMIdx = kGroupM * band + rem % bandTiles;
+    t.valid = 1;
+    t.group = lo;
+    t.tileN = rem / bandTiles;
+    t.rowBase = rowStartTbl[lo] + tileMIdx * kTileM;
+    t.rows = min(kTileM, rowCountTbl[lo] - tileMIdx * kTileM);  // >= 1
+    t.colBase = kSwiglu ? t.tileN * (kTileN / 2) : t.tileN * kTileN;
+    return t;
+}
+
+// Output channel held in row r of the weight tile (clamped: channels past N are loaded but never stored).
+template <bool kSwiglu>
+__device__ __forceinline__ int32_t ChannelOfRow(const KernelArgs& a, const TileInfo& t, int r) {
+    int32_t n;
+    if (kSwiglu) n = r < kTileN / 2 ? t.colBase + r : a.halfN + t.colBase + (r - kTileN / 2);
+    else n = t.colBase + r;
+    return n < a.N ? n : a.N - 1;
+}
 
 __device__ __forceinline__ float LoadScale(const void* p, int64_t i, int dtype) {
     if (dtype == 0) return static_cast<const float*>(p)[i];
@@ -158,208 +202,25 @@ __device__ __forceinline__ uint16_t ToBf16(float f) {
     return static_cast<uint16_t>(u >> 16);
 }
 
-// kFastLoad: 16-byte global loads (K-contiguous weights, K % 16 == 0, 16-byte aligned bases).  Otherwise byte-wise.
-template <int kSubM, int kWavesM, Epilogue kEpi, bool kFastLoad>
-__global__ __launch_bounds__(256 * kWavesM) void GroupedGemmKernel(KernelArgs a) {
-    constexpr int kThreads = 256 * kWavesM;
-    constexpr int kTileM = 32 * kSubM * kWavesM;
-    constexpr int kRowsPerPass = kThreads / kChunksPerRow;  // tile rows covered by one load per thread
-    constexpr int kALoads = kTileM / kRowsPerPass;           // == kSubM
-    constexpr int kBLoads = kTileN / kRowsPerPass;
-    constexpr bool kSwiglu = kEpi == Epilogue::kSwiglu;
-    extern __shared__ __attribute__((aligned(16))) char lds[];
-    char* const ldsA = lds;
-    char* const ldsB = lds + 2 * kTileM * kStepBytes;
-
-    // ---- which tile ----
-    const int32_t totalMTiles = a.sched[1];
-    const int64_t totalTiles = static_cast<int64_t>(totalMTiles) * a.tilesN;
-    const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
-    const int64_t local = blockIdx.x / kXcds;
-    const int64_t logical = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd + local;
-    if (local >= perXcd || logical >= totalTiles) return;
-    const int32_t* rowStartTbl = a.sched + 2;
-    const int32_t* rowCountTbl = rowStartTbl + a.groups;
-    const int32_t* tilePrefix = rowCountTbl + a.groups;
-    const int32_t q = static_cast<int32_t>(logical / a.tilesN);
-    int lo = 0, hi = a.groups;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (tilePrefix[mid] <= q) lo = mid; else hi = mid;
-    }
-    const int group = lo;
-    const int32_t inGroup = static_cast<int32_t>(logical - static_cast<int64_t>(tilePrefix[group]) * a.tilesN);
-    const int32_t tilesM = tilePrefix[group + 1] - tilePrefix[group];
-    const int32_t band = inGroup / (kGroupM * a.tilesN);
-    const int32_t rem = inGroup % (kGroupM * a.tilesN);
-    const int32_t bandTiles = min(kGroupM, tilesM - kGroupM * band);
-    const int32_t tileN = rem / bandTiles;
-    const int32_t tileMIdx = kGroupM * band + rem % bandTiles;
-    const int32_t rowBase = rowStartTbl[group] + tileMIdx * kTileM;
-    const int32_t rows = min(kTileM, rowCountTbl[group] - tileMIdx * kTileM);  // >= 1
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int waveN = wave % kWavesN;
-    const int waveM = wave / kWavesN;
-    const int l32 = lane & 31;
-    const int lhi = lane >> 5;
-
-    // Output channel held in LDS row r of the weight tile.
-    const int32_t colBase = kSwiglu ? tileN * (kTileN / 2) : tileN * kTileN;
-    auto channelOfRow = [&](int r) -> int32_t {
-        int32_t n;
-        if (kSwiglu) n = r < kTileN / 2 ? colBase + r : a.halfN + colBase + (r - kTileN / 2);
-        else n = colBase + r;
-        return n < a.N ? n : a.N - 1;  // clamped loads; such columns are never stored
-    };
-
-    const int8_t* const wGroup = a.w + static_cast<int64_t>(group) * a.wGroupStride;
-    const int kSteps = (a.K + kStepBytes - 1) / kStepBytes;
-
-    v4i regA[kALoads];
-    v4i regB[kBLoads];
-
-    auto loadGlobal = [&](int step) {
-        const int k0 = step * kStepBytes;
-        if (kFastLoad) {
-            const int chunk = tid % kChunksPerRow;
-            const int rowInPass = tid / kChunksPerRow;
-            const int k = k0 + chunk * kChunk;
-            const bool kValid = k < a.K;
-#pragma unroll
-            for (int i = 0; i < kALoads; ++i) {
-                const int r = i * kRowsPerPass + rowInPass;
-                v4i v = {0, 0, 0, 0};
-                if (i * kRowsPerPass < rows && kValid) {
-                    const int rr = r < rows ? r : rows - 1;
-                    v = *reinterpret_cast<const v4i*>(a.x + static_cast<int64_t>(rowBase + rr) * a.K + k);
-                }
-                regA[i] = v;
-            }
-#pragma unroll
-            for (int i = 0; i < kBLoads; ++i) {
-                const int r = i * kRowsPerPass + rowInPass;
-                v4i v = {0, 0, 0, 0};
-                if (kValid) v = *reinterpret_cast<const v4i*>(wGroup + static_cast<int64_t>(channelOfRow(r)) * a.wStrideN + k);
-                regB[i] = v;
-            }
-        } else {
-            // byte-wise: consecutive threads take consecutive tile rows so that N-contiguous weights still coalesce
-#pragma unroll
-            for (int i = 0; i < kALoads; ++i) {
-                const int p = i * kThreads + tid;
-                const int r = p % kTileM;
-                const int chunk = p / kTileM;
-                const int rr = r < rows ? r : rows - 1;
-                const int8_t* src = a.x + static_cast<int64_t>(rowBase + rr) * a.K;
-                union { v4i v; int8_t b[16]; } u;
-                for (int j = 0; j < kChunk; ++j) {
-                    const int k = k0 + chunk * kChunk + j;
-                    u.b[j] = k < a.K ? src[k] : static_cast<int8_t>(0);
-                }
-                regA[i] = u.v;
-            }
-#pragma unroll
-            for (int i = 0; i < kBLoads; ++i) {
-                const int p = i * kThreads + tid;
-                const int r = p % kTileN;
-                const int chunk = p / kTileN;
-                const int8_t* src = wGroup + static_cast<int64_t>(channelOfRow(r)) * a.wStrideN;
-                union { v4i v; int8_t b[16]; } u;
-                for (int j = 0; j < kChunk; ++j) {
-                    const int k = k0 + chunk * kChunk + j;
-                    u.b[j] = k < a.K ? src[static_cast<int64_t>(k) * a.wStrideK] : static_cast<int8_t>(0);
-                }
-                regB[i] = u.v;
-            }
-        }
-    };
-
-    auto storeLds = [&](int buf) {
-        char* A = ldsA + buf * kTileM * kStepBytes;
-        char* B = ldsB + buf * kTileN * kStepBytes;
-        if (kFastLoad) {
-            const int chunk = tid % kChunksPerRow;
-            const int rowInPass = tid / kChunksPerRow;
-#pragma unroll
-            for (int i = 0; i < kALoads; ++i) {
-                const int r = i * kRowsPerPass + rowInPass;
-                *reinterpret_cast<v4i*>(A + LdsOffset(r, chunk)) = regA[i];
-            }
-#pragma unroll
-            for (int i = 0; i < kBLoads; ++i) {
-                const int r = i * kRowsPerPass + rowInPass;
-                *reinterpret_cast<v4i*>(B + LdsOffset(r, chunk)) = regB[i];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < kALoads; ++i) {
-                const int p = i * kThreads + tid;
-                *reinterpret_cast<v4i*>(A + LdsOffset(p % kTileM, p / kTileM)) = regA[i];
-            }
-#pragma unroll
-            for (int i = 0; i < kBLoads; ++i) {
-                const int p = i * kThreads + tid;
-                *reinterpret_cast<v4i*>(B + LdsOffset(p % kTileN, p / kTileN)) = regB[i];
-            }
-        }
-    };
-
-    // ---- main loop ----
-    v16i acc[kSubM][2];
-#pragma unroll
-    for (int mi = 0; mi < kSubM; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
-
-    const int waveRow0 = waveM * 32 * kSubM;
-    int active = (rows - waveRow0 + 31) / 32;  // 32-row MFMA tiles of this wave that hold real rows
-    active = active < 0 ? 0 : (active > kSubM ? kSubM : active);
-    const int bRow0 = kSwiglu ? 32 * waveN : 64 * waveN;
-    const int bRowStep = kSwiglu ? kTileN / 2 : 32;
-
-    loadGlobal(0);
-    storeLds(0);
-    __syncthreads();
-    for (int step = 0; step < kSteps; ++step) {
-        const int buf = step & 1;
-        if (step + 1 < kSteps) loadGlobal(step + 1);
-        const char* A = ldsA + buf * kTileM * kStepBytes;
-        const char* B = ldsB + buf * kTileN * kStepBytes;
-#pragma unroll
-        for (int ks = 0; ks < kStepBytes / 32; ++ks) {
-            const int chunk = 2 * ks + lhi;
-            const v4i b0 = *reinterpret_cast<const v4i*>(B + LdsOffset(bRow0 + l32, chunk));
-            const v4i b1 = *reinterpret_cast<const v4i*>(B + LdsOffset(bRow0 + bRowStep + l32, chunk));
-#pragma unroll
-            for (int mi = 0; mi < kSubM; ++mi) {
-                if (mi < active) {
-                    const v4i av = *reinterpret_cast<const v4i*>(A + LdsOffset(waveRow0 + mi * 32 + l32, chunk));
-                    acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b0, acc[mi][0], 0, 0, 0);
-                    acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, acc[mi][1], 0, 0, 0);
-                }
-            }
-        }
-        if (step + 1 < kSteps) storeLds(buf ^ 1);
-        __syncthreads();
-    }
-
-    // ---- epilogue ----
-    // acc[mi][ni][v] is C[row, col] with row = waveRow0 + 32*mi + 8*(v/4) + 4*lhi + (v%4), col = column block ni, lane l32.
+// Epilogue of one tile.  acc[mi][ni][v] is C[row, col] with row = waveRow0 + 32*mi + 8*(v/4) + 4*lhi + (v%4); the wave
+// owns column blocks ni = 0, 1, lane l32 inside each (plain: 64*waveN + 32*ni; kSwiglu: S column 32*waveN and its partner).
+// ldsRowScale holds the tile's per-row scales.  Contains workgroup barriers: every wave must call it.
+template <int kSubM, int kTileM, Epilogue kEpi>
+__device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo& t, v16i (&acc)[kSubM][2], int waveRow0,
+                                             int waveN, int l32, int lhi, int tid, const float* ldsRowScale,
+                                             float* ldsRowMax) {
+    const int32_t rows = t.rows, rowBase = t.rowBase, group = t.group;
     if (kEpi == Epilogue::kInt32 || kEpi == Epilogue::kDequant) {
+        const bool hasRowScale = a.rowScale != nullptr;
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni) {
-            const int32_t n = colBase + 64 * waveN + 32 * ni + l32;
+            const int32_t n = t.colBase + 64 * waveN + 32 * ni + l32;
             const bool nValid = n < a.N;
             float sc = 0.0f;
             if (kEpi == Epilogue::kDequant && nValid) sc = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + n, a.scaleDtype);
 #pragma unroll
             for (int mi = 0; mi < kSubM; ++mi) {
-                if (mi >= active) continue;
+                if (waveRow0 + 32 * mi >= rows) continue;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int r = waveRow0 + 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
@@ -369,7 +230,7 @@ __global__ __launch_bounds__(256 * kWavesM) void GroupedGemmKernel(KernelArgs a)
                         static_cast<int32_t*>(a.out)[o] = acc[mi][ni][v];
                     } else {
                         float y = __fmul_rn(static_cast<float>(acc[mi][ni][v]), sc);
-                        if (a.rowScale != nullptr) y = __fmul_rn(y, a.rowScale[rowBase + r]);
+                        if (hasRowScale) y = __fmul_rn(y, ldsRowScale[r]);
                         if (a.outDtype == 27) static_cast<uint16_t*>(a.out)[o] = ToBf16(y);
                         else if (a.outDtype == 1) static_cast<__half*>(a.out)[o] = __float2half_rn(y);
                         else static_cast<float*>(a.out)[o] = y;
@@ -378,7 +239,7 @@ __global__ __launch_bounds__(256 * kWavesM) void GroupedGemmKernel(KernelArgs a)
             }
         }
     } else {
-        const int32_t j = colBase + 32 * waveN + l32;  // column of S
+        const int32_t j = t.colBase + 32 * waveN + l32;  // column of S
         const bool jValid = j < a.halfN;
         float scA = 0.0f, scB = 0.0f;
         if (jValid) {
@@ -387,32 +248,326 @@ __global__ __launch_bounds__(256 * kWavesM) void GroupedGemmKernel(KernelArgs a)
         }
 #pragma unroll
         for (int mi = 0; mi < kSubM; ++mi) {
-            if (mi >= active) continue;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int r = waveRow0 + 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
                 const bool valid = r < rows && jValid;
                 float s = 0.0f;
                 if (valid) {
-                    const float xs = a.rowScale[rowBase + r];
+                    const float xs = ldsRowScale[r];
                     const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), xs), scA);
                     const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xs), scB);
                     s = __fmul_rn(__fdiv_rn(ca, __fadd_rn(1.0f, expf(-ca))), cb);
                     a.sOut[static_cast<int64_t>(rowBase + r) * a.halfN + j] = s;
                 }
+                // max |S| of this row over the wave's 32 columns, kept by the first lane of each half-wave
                 float m = fabsf(s);
 #pragma unroll
                 for (int d = 1; d < 32; d <<= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
-                if (l32 == 0 && r < rows) atomicMax(a.rowMax + rowBase + r, __float_as_uint(m));
+                if (l32 == 0) ldsRowMax[waveN * kTileM + r] = m;
             }
         }
+        __syncthreads();
+        // one partial maximum per (n-tile, row): no atomics and nothing to pre-zero; the requantisation folds them
+        if (tid < rows) {
+            float m = ldsRowMax[tid];
+#pragma unroll
+            for (int w = 1; w < kWavesN; ++w) m = fmaxf(m, ldsRowMax[w * kTileM + tid]);
+            a.rowMax[static_cast<int64_t>(t.tileN) * a.M + rowBase + tid] = m;
+        }
     }
+}
+
+// ---------------------------------------------------------------------------------------------- fast path: LDS-DMA ring
+constexpr int kDmaStep = 64;  // k-bytes per ring stage
+
+template <int kSubM, int kWavesM>
+struct StreamCfg {
+    static constexpr int kWaves = kWavesN * kWavesM;
+    static constexpr int kThreads = 64 * kWaves;
+    static constexpr int kTileM = 32 * kSubM * kWavesM;
+    static constexpr int kStageBytes = (kTileM + kTileN) * kDmaStep;
+    static constexpr int kScratchBytes = (1 + kWavesN) * kTileM * 4;
+    static constexpr int kStagesFit = (kLdsBudget - kScratchBytes) / kStageBytes;
+    static constexpr int kStages = kStagesFit > 8 ? 8 : kStagesFit;
+    static constexpr int kLdsBytes = kStages * kStageBytes + kScratchBytes;
+    // one DMA instruction moves 64 lanes x 16 bytes = 16 rows of 64 k-bytes
+    static constexpr int kInstrA = kTileM * kDmaStep / 1024;
+    static constexpr int kInstr = (kTileM + kTileN) * kDmaStep / 1024;
+    static constexpr int kMaxPerWave = (kInstr + kWaves - 1) / kWaves;
+    static_assert(kStages >= 3, "the ring needs at least three stages");
+    static_assert((kStages - 2) * kMaxPerWave <= 63, "vmcnt is a 6-bit counter");
+};
+
+__device__ __forceinline__ int Lds64Offset(int row, int chunk) { return row * kDmaStep + ((chunk ^ ((row >> 2) & 3)) << 4); }
+
+// 16 bytes per lane from (uniform base + 32-bit lane offset) straight into LDS at ldsDst + lane * 16.  The compiler does
+// not see this as a memory instruction: completion is awaited with WaitVmcnt below.
+__device__ __forceinline__ void DmaToLds16(const char* base, uint32_t laneOffset, char* ldsDst) {
+    typedef __attribute__((address_space(3))) char* LdsPtr;  // the 32-bit LDS address of a generic pointer into LDS
+    const uint32_t m0 = static_cast<uint32_t>(
+        __builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(reinterpret_cast<size_t>((LdsPtr)ldsDst)))));
+    // The base is wave-uniform by construction; readfirstlane makes the compiler keep it in scalar registers.
+    // readfirstlane returns a signed int: each half is widened through uint32_t so that a low word with its top bit
+    // set cannot sign-extend into the high word.
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(b))));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(b >> 32))));
+    const uint64_t sbase = static_cast<uint64_t>(lo) | (static_cast<uint64_t>(hi) << 32);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(laneOffset), "s"(sbase) : "memory");
+}
+
+template <int kCount>
+__device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leaving expcnt / lgkmcnt untouched
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (kCount & 15) | ((kCount >> 4) << 14));
+}
+
+// Persistent: the grid is one workgroup per CU (a multiple of 8); workgroup b serves XCD b % 8 and walks that XCD's
+// share of the tile list with stride gridDim / 8.
+template <int kSubM, int kWavesM, Epilogue kEpi>
+__global__ __launch_bounds__(256 * kWavesM) void StreamGemmKernel(KernelArgs a) {
+    using Cfg = StreamCfg<kSubM, kWavesM>;
+    constexpr int kTileM = Cfg::kTileM;
+    constexpr int kStages = Cfg::kStages;
+    constexpr int kStageBytes = Cfg::kStageBytes;
+    constexpr bool kSwiglu = kEpi == Epilogue::kSwiglu;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    float* const ldsRowScale = reinterpret_cast<float*>(lds + kStages * kStageBytes);  // [kTileM]
+    float* const ldsRowMax = ldsRowScale + kTileM;                                      // [kWavesN][kTileM]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waveN = wave % kWavesN;
+    const int waveM = wave / kWavesN;
+    const int l32 = lane & 31;
+    const int lhi = lane >> 5;
+
+    const int64_t totalTiles = static_cast<int64_t>(a.sched[1]) * a.tilesN;
+    const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
+    const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
+    const int64_t slots = gridDim.x / kXcds;
+    auto decode = [&](int64_t local) { return DecodeTile<kTileM, kSwiglu>(a, xcdFirst, perXcd, totalTiles, local); };
+
+    int64_t local = blockIdx.x / kXcds;
+    TileInfo cur = decode(local);
+    if (!cur.valid) return;
+    const int kSteps = a.K / kDmaStep;
+
+    // ---- issue side: runs kStages - 1 steps ahead of the compute side, across tile boundaries ----
+    TileInfo iss = cur;
+    int64_t issLocal = local;
+    int issStep = 0;
+    const char* issX = nullptr;
+    const char* issW = nullptr;
+    uint32_t laneOff[Cfg::kMaxPerWave];
+    int dmaPerStage = 0;  // DMA instructions this wave issues per stage
+#pragma unroll
+    for (int q = 0; q < Cfg::kMaxPerWave; ++q) dmaPerStage += (wave + q * Cfg::kWaves < Cfg::kInstr) ? 1 : 0;
+
+    auto setupIssue = [&]() {
+        issX = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(iss.rowBase) * a.K;
+        issW = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(iss.group) * a.wGroupStride;
+        const int rowLimit = a.M - 1 - iss.rowBase;  // rows past the tile read whatever follows in x, never beyond it
+        const int rowIn = lane >> 2;
+        const int slot = lane & 3;
+#pragma unroll
+        for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
+            const int j = wave + q * Cfg::kWaves;
+            if (j < Cfg::kInstrA) {
+                const int r = 16 * j + rowIn;
+                const int c = slot ^ ((r >> 2) & 3);
+                laneOff[q] = static_cast<uint32_t>(min(r, rowLimit) * a.K + c * kChunk);
+            } else {
+                const int r = 16 * (j - Cfg::kInstrA) + rowIn;
+                const int c = slot ^ ((r >> 2) & 3);
+                laneOff[q] = static_cast<uint32_t>(ChannelOfRow<kSwiglu>(a, iss, r) * a.K + c * kChunk);
+            }
+        }
+    };
+    auto issueStage = [&](int ring) {
+        char* const dst = lds + ring * kStageBytes;
+        const int kOff = issStep * kDmaStep;
+#pragma unroll
+        for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
+            const int j = wave + q * Cfg::kWaves;
+            if (j < Cfg::kInstr) DmaToLds16((j < Cfg::kInstrA ? issX : issW) + kOff, laneOff[q], dst + j * 1024);
+        }
+        if (++issStep == kSteps) {
+            // move to this workgroup's next tile; past the last one the same tile is fetched again into ring slots
+            // nobody reads, which keeps the number of outstanding DMAs per stage constant
+            issStep = 0;
+            const TileInfo next = decode(issLocal + slots);
+            if (next.valid) {
+                iss = next;
+                issLocal += slots;
+            }
+            setupIssue();
+        }
+    };
+
+    setupIssue();
+#pragma unroll 1
+    for (int s = 0; s < kStages - 1; ++s) issueStage(s);
+    int ring = 0;  // stage the compute side reads next; the issue side writes (ring + kStages - 1) % kStages
+
+    if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
+        ldsRowScale[tid] = a.rowScale[cur.rowBase + (tid < cur.rows ? tid : cur.rows - 1)];
+    }
+
+    const int waveRow0 = waveM * 32 * kSubM;
+    const int bRow0 = kSwiglu ? 32 * waveN : 64 * waveN;
+    const int bRowStep = kSwiglu ? kTileN / 2 : 32;
+    v16i acc[kSubM][2];
+
+    while (true) {
+        const TileInfo following = decode(local + slots);
+        // the next tile's per-row scale travels in a register until this tile's epilogue has read the LDS copy
+        float followingRowScale = 0.0f;
+        if (following.valid && kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
+            followingRowScale = a.rowScale[following.rowBase + (tid < following.rows ? tid : following.rows - 1)];
+        }
+#pragma unroll
+        for (int mi = 0; mi < kSubM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
+
+#pragma unroll 1
+        for (int step = 0; step < kSteps; ++step) {
+            // the oldest stage in flight has landed once at most (kStages - 2) stages' worth of this wave's DMAs remain
+            if (dmaPerStage == Cfg::kMaxPerWave) WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
+            else WaitVmcnt<(kStages - 2) * (Cfg::kMaxPerWave - 1)>();
+            __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
+            issueStage(ring == 0 ? kStages - 1 : ring - 1);
+            const char* const A = lds + ring * kStageBytes;
+            const char* const B = A + kTileM * kDmaStep;
+#pragma unroll
+            for (int ks = 0; ks < kDmaStep / 32; ++ks) {
+                const int chunk = 2 * ks + lhi;
+                const v4i b0 = *reinterpret_cast<const v4i*>(B + Lds64Offset(bRow0 + l32, chunk));
+                const v4i b1 = *reinterpret_cast<const v4i*>(B + Lds64Offset(bRow0 + bRowStep + l32, chunk));
+#pragma unroll
+                for (int mi = 0; mi < kSubM; ++mi) {
+                    const v4i av = *reinterpret_cast<const v4i*>(A + Lds64Offset(waveRow0 + mi * 32 + l32, chunk));
+                    acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b0, acc[mi][0], 0, 0, 0);
+                    acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, acc[mi][1], 0, 0, 0);
+                }
+            }
+            ring = ring + 1 == kStages ? 0 : ring + 1;
+        }
+
+        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, waveRow0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
+        // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
+        // stores and the DMAs in flight, which had the whole epilogue to land) before counting DMAs again.
+        WaitVmcnt<0>();
+        if (!following.valid) break;
+        __syncthreads();  // the epilogue's reads of ldsRowScale / ldsRowMax are done
+        if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) ldsRowScale[tid] = followingRowScale;
+        cur = following;
+        local += slots;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------- generic path
+constexpr int kGenStep = 128;  // k-bytes per step
+
+__device__ __forceinline__ int Lds128Offset(int row, int chunk) { return row * kGenStep + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+// One tile per workgroup (grid = static upper bound of tiles), 4 waves, operands gathered byte by byte through
+// registers into a single LDS buffer.  Handles any K and both weight layouts.
+template <int kSubM, Epilogue kEpi>
+__global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a) {
+    constexpr int kThreads = 256;
+    constexpr int kTileM = 32 * kSubM;
+    constexpr int kChunksPerRow = kGenStep / kChunk;
+    constexpr int kALoads = kTileM * kChunksPerRow / kThreads;
+    constexpr int kBLoads = kTileN * kChunksPerRow / kThreads;
+    constexpr bool kSwiglu = kEpi == Epilogue::kSwiglu;
+    __shared__ __attribute__((aligned(16))) char ldsA[kTileM * kGenStep];
+    __shared__ __attribute__((aligned(16))) char ldsB[kTileN * kGenStep];
+    __shared__ float ldsRowScale[kTileM];
+    __shared__ float ldsRowMax[kWavesN * kTileM];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int waveN = tid >> 6;
+    const int l32 = lane & 31;
+    const int lhi = lane >> 5;
+
+    const int64_t totalTiles = static_cast<int64_t>(a.sched[1]) * a.tilesN;
+    const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
+    const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
+    const TileInfo t = DecodeTile<kTileM, kSwiglu>(a, xcdFirst, perXcd, totalTiles, blockIdx.x / kXcds);
+    if (!t.valid) return;
+    if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
+        ldsRowScale[tid] = a.rowScale[t.rowBase + (tid < t.rows ? tid : t.rows - 1)];
+    }
+    const int8_t* const wGroup = a.w + static_cast<int64_t>(t.group) * a.wGroupStride;
+    const int bRow0 = kSwiglu ? 32 * waveN : 64 * waveN;
+    const int bRowStep = kSwiglu ? kTileN / 2 : 32;
+
+    v16i acc[kSubM][2];
+#pragma unroll
+    for (int mi = 0; mi < kSubM; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
+
+    for (int k0 = 0; k0 < a.K; k0 += kGenStep) {
+        // consecutive threads take consecutive tile rows so that N-contiguous weights still coalesce
+#pragma unroll
+        for (int i = 0; i < kALoads; ++i) {
+            const int p = i * kThreads + tid;
+            const int r = p % kTileM;
+            const int chunk = p / kTileM;
+            const int8_t* src = a.x + static_cast<int64_t>(t.rowBase + (r < t.rows ? r : t.rows - 1)) * a.K;
+            union { v4i v; int8_t b[16]; } u;
+            for (int j = 0; j < kChunk; ++j) {
+                const int k = k0 + chunk * kChunk + j;
+                u.b[j] = k < a.K ? src[k] : static_cast<int8_t>(0);
+            }
+            *reinterpret_cast<v4i*>(ldsA + Lds128Offset(r, chunk)) = u.v;
+        }
+#pragma unroll
+        for (int i = 0; i < kBLoads; ++i) {
+            const int p = i * kThreads + tid;
+            const int r = p % kTileN;
+            const int chunk = p / kTileN;
+            const int8_t* src = wGroup + static_cast<int64_t>(ChannelOfRow<kSwiglu>(a, t, r)) * a.wStrideN;
+            union { v4i v; int8_t b[16]; } u;
+            for (int j = 0; j < kChunk; ++j) {
+                const int k = k0 + chunk * kChunk + j;
+                u.b[j] = k < a.K ? src[static_cast<int64_t>(k) * a.wStrideK] : static_cast<int8_t>(0);
+            }
+            *reinterpret_cast<v4i*>(ldsB + Lds128Offset(r, chunk)) = u.v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < kGenStep / 32; ++ks) {
+            const int chunk = 2 * ks + lhi;
+            const v4i b0 = *reinterpret_cast<const v4i*>(ldsB + Lds128Offset(bRow0 + l32, chunk));
+            const v4i b1 = *reinterpret_cast<const v4i*>(ldsB + Lds128Offset(bRow0 + bRowStep + l32, chunk));
+#pragma unroll
+            for (int mi = 0; mi < kSubM; ++mi) {
+                const v4i av = *reinterpret_cast<const v4i*>(ldsA + Lds128Offset(mi * 32 + l32, chunk));
+                acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b0, acc[mi][0], 0, 0, 0);
+                acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, acc[mi][1], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    TileEpilogue<kSubM, kTileM, kEpi>(a, t, acc, 0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
 }
 
 // ---------------------------------------------------------------------------------------------- requantisation
 struct RequantArgs {
     const float* s;          // [M, halfN]
-    const uint32_t* rowMax;  // [M] bit pattern of max |S|
+    const float* rowMax;     // [tilesN][M] partial max |S|
+    int32_t tilesN;
+    int64_t M;
     const int32_t* sched;
     int8_t* y;               // [M, halfN]
     float* yScale;           // [M]
@@ -428,7 +583,16 @@ __device__ __forceinline__ int8_t QuantOne(float s, float inv) {
 __global__ __launch_bounds__(256) void RequantKernel(RequantArgs a) {
     const int64_t row = blockIdx.x;
     if (row >= a.sched[0]) return;
-    const float mx = __uint_as_float(a.rowMax[row]);
+    __shared__ float rowMaxShared;
+    if (threadIdx.x < 64) {  // the first wave folds the per-n-tile partial maxima
+        float m = 0.0f;
+        for (int t = threadIdx.x; t < a.tilesN; t += 64) m = fmaxf(m, a.rowMax[static_cast<int64_t>(t) * a.M + row]);
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
+        if (threadIdx.x == 0) rowMaxShared = m;
+    }
+    __syncthreads();
+    const float mx = rowMaxShared;
     const float ys = __fdiv_rn(mx, 127.0f);
     const float inv = __fdiv_rn(1.0f, ys);
     if (threadIdx.x == 0) a.yScale[row] = ys;
@@ -451,38 +615,56 @@ __global__ __launch_bounds__(256) void RequantKernel(RequantArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------- dispatch
-template <int kSubM, int kWavesM, Epilogue kEpi, bool kFastLoad>
-hipError_t LaunchOne(const KernelArgs& args, int64_t grid, hipStream_t stream) {
-    constexpr int kTileM = 32 * kSubM * kWavesM;
-    constexpr int kLdsBytes = 2 * (kTileM + kTileN) * kStepBytes;
-    auto kernel = GroupedGemmKernel<kSubM, kWavesM, kEpi, kFastLoad>;
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+int DeviceCuCount() {
+    static const int count = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+        return n;
+    }();
+    return count;
+}
+
+template <int kSubM, int kWavesM, Epilogue kEpi>
+hipError_t LaunchStream(const KernelArgs& args, int64_t maxTiles, hipStream_t stream) {
+    using Cfg = StreamCfg<kSubM, kWavesM>;
+    auto kernel = StreamGemmKernel<kSubM, kWavesM, kEpi>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
     if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(256 * kWavesM), kLdsBytes, stream, args);
+    // persistent grid: one workgroup per CU (the LDS ring fills the CU), a multiple of the XCD count
+    int64_t grid = DeviceCuCount();
+    if (grid > maxTiles) grid = maxTiles;
+    grid = grid / kXcds * kXcds;
+    if (grid < kXcds) grid = kXcds;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, args);
     return hipGetLastError();
 }
 
-template <Epilogue kEpi, bool kFastLoad>
-hipError_t LaunchShape(const Plan& plan, const KernelArgs& args, int64_t grid, hipStream_t stream) {
-    if constexpr (!kFastLoad) {  // the byte-wise loader exists for two shapes only
-        if (plan.tileM <= 32) return LaunchOne<1, 1, kEpi, false>(args, grid, stream);
-        return LaunchOne<4, 1, kEpi, false>(args, grid, stream);
-    } else {
-        switch (plan.tileM) {
-            case 32: return LaunchOne<1, 1, kEpi, true>(args, grid, stream);
-            case 64: return LaunchOne<2, 1, kEpi, true>(args, grid, stream);
-            case 96: return LaunchOne<3, 1, kEpi, true>(args, grid, stream);
-            case 128: return LaunchOne<4, 1, kEpi, true>(args, grid, stream);
-            case 192: return LaunchOne<3, 2, kEpi, true>(args, grid, stream);
-            default: return LaunchOne<4, 2, kEpi, true>(args, grid, stream);
-        }
+template <Epilogue kEpi>
+hipError_t LaunchStreamShape(const Plan& plan, const KernelArgs& args, hipStream_t stream) {
+    switch (plan.tileM) {
+        case 32: return LaunchStream<1, 1, kEpi>(args, plan.maxTiles, stream);
+        case 64: return LaunchStream<1, 2, kEpi>(args, plan.maxTiles, stream);
+        case 128: return LaunchStream<2, 2, kEpi>(args, plan.maxTiles, stream);
+        case 192: return LaunchStream<3, 2, kEpi>(args, plan.maxTiles, stream);
+        default: return LaunchStream<4, 2, kEpi>(args, plan.maxTiles, stream);
     }
 }
 
-bool FastLoadOk(const Problem& p) {
-    return p.wKMajor && p.K % kChunk == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
-           reinterpret_cast<uintptr_t>(p.w) % kChunk == 0;
+template <Epilogue kEpi>
+hipError_t LaunchGenericShape(const Plan& plan, const KernelArgs& args, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>(plan.maxTiles));
+    if (plan.tileM <= 32) hipLaunchKernelGGL((GenericGemmKernel<1, kEpi>), grid, dim3(256), 0, stream, args);
+    else hipLaunchKernelGGL((GenericGemmKernel<4, kEpi>), grid, dim3(256), 0, stream, args);
+    return hipGetLastError();
+}
+
+// The DMA ring needs K-contiguous weights, whole 64-byte k steps, 16-byte aligned bases and 32-bit offsets inside one
+// expert's weights.
+bool StreamOk(const Problem& p) {
+    return p.wKMajor && p.K % kDmaStep == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
+           reinterpret_cast<uintptr_t>(p.w) % kChunk == 0 && p.N * p.K < (1ll << 31);
 }
 
 uint64_t Align256(uint64_t v) { return (v + 255) / 256 * 256; }
@@ -493,13 +675,16 @@ Plan MakePlan(const Problem& p) {
     Plan plan;
     const int64_t groups = p.groups > 0 ? p.groups : 1;
     const double want = static_cast<double>(p.M) / static_cast<double>(groups) * 1.3;
-    static const int kShapes[] = {32, 64, 96, 128, 192, 256};
-    plan.tileM = 256;
-    for (int s : kShapes) {
-        if (static_cast<double>(s) >= want) { plan.tileM = s; break; }
+    if (StreamOk(p)) {
+        static const int kShapes[] = {32, 64, 128, 192, 256};
+        plan.tileM = 256;
+        for (int s : kShapes) {
+            if (static_cast<double>(s) >= want) { plan.tileM = s; break; }
+        }
+    } else {
+        plan.tileM = want <= 32.0 ? 32 : 128;
     }
-    if (!FastLoadOk(p)) plan.tileM = plan.tileM <= 32 ? 32 : 128;
-    plan.wavesM = plan.tileM > 128 ? 2 : 1;
+    plan.wavesM = plan.tileM >= 64 && StreamOk(p) ? 2 : 1;
     plan.subTilesM = plan.tileM / 32 / plan.wavesM;
     const int64_t cols = p.epilogue == Epilogue::kSwiglu ? p.N / 2 : p.N;
     const int64_t colsPerTile = p.epilogue == Epilogue::kSwiglu ? kTileN / 2 : kTileN;
@@ -512,7 +697,7 @@ Plan MakePlan(const Problem& p) {
     off += Align256(static_cast<uint64_t>(SchedInts(static_cast<int>(groups))) * 4);
     if (p.epilogue == Epilogue::kSwiglu) {
         plan.offRowMax = off;
-        off += Align256(static_cast<uint64_t>(p.M) * 4);
+        off += Align256(static_cast<uint64_t>(p.M) * 4 * static_cast<uint64_t>(plan.tilesN));
         plan.offS = off;
         off += Align256(static_cast<uint64_t>(p.M) * static_cast<uint64_t>(p.N / 2) * 4);
     }
@@ -526,13 +711,12 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     char* ws = static_cast<char*>(workspace);
     int32_t* sched = reinterpret_cast<int32_t*>(ws + plan.offSched);
     const bool swiglu = p.epilogue == Epilogue::kSwiglu;
-    uint32_t* rowMax = swiglu ? reinterpret_cast<uint32_t*>(ws + plan.offRowMax) : nullptr;
+    float* rowMax = swiglu ? reinterpret_cast<float*>(ws + plan.offRowMax) : nullptr;
     float* sBuf = swiglu ? reinterpret_cast<float*>(ws + plan.offS) : nullptr;
 
     SchedArgs sa{};
     sa.groupList = p.groupList;
     sa.sched = sched;
-    sa.rowMax = rowMax;
     sa.groups = p.groups;
     sa.groupListIsInt64 = p.groupListIsInt64 ? 1 : 0;
     sa.isCount = p.groupListKind == GroupListKind::kCount ? 1 : 0;
@@ -566,27 +750,27 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
 
     hipError_t e = hipSuccess;
     if (p.K > 0) {
-        const bool fast = FastLoadOk(p);
+        const bool fast = StreamOk(p);
         opapi::KernelTimer timer(p.epilogue == Epilogue::kSwiglu ? "gmm_swiglu"
                                  : p.epilogue == Epilogue::kDequant ? "gmm_dequant" : "gmm_int32", stream);
         switch (p.epilogue) {
             case Epilogue::kInt32:
-                e = fast ? LaunchShape<Epilogue::kInt32, true>(plan, ka, plan.maxTiles, stream)
-                         : LaunchShape<Epilogue::kInt32, false>(plan, ka, plan.maxTiles, stream);
+                e = fast ? LaunchStreamShape<Epilogue::kInt32>(plan, ka, stream)
+                         : LaunchGenericShape<Epilogue::kInt32>(plan, ka, stream);
                 break;
             case Epilogue::kDequant:
-                e = fast ? LaunchShape<Epilogue::kDequant, true>(plan, ka, plan.maxTiles, stream)
-                         : LaunchShape<Epilogue::kDequant, false>(plan, ka, plan.maxTiles, stream);
+                e = fast ? LaunchStreamShape<Epilogue::kDequant>(plan, ka, stream)
+                         : LaunchGenericShape<Epilogue::kDequant>(plan, ka, stream);
                 break;
             case Epilogue::kSwiglu:
-                e = fast ? LaunchShape<Epilogue::kSwiglu, true>(plan, ka, plan.maxTiles, stream)
-                         : LaunchShape<Epilogue::kSwiglu, false>(plan, ka, plan.maxTiles, stream);
+                e = fast ? LaunchStreamShape<Epilogue::kSwiglu>(plan, ka, stream)
+                         : LaunchGenericShape<Epilogue::kSwiglu>(plan, ka, stream);
                 break;
         }
         if (e != hipSuccess) return e;
     }
     if (swiglu) {
-        RequantArgs ra{sBuf, rowMax, sched, p.quantOut, p.quantScaleOut, static_cast<int32_t>(p.N / 2)};
+        RequantArgs ra{sBuf, rowMax, plan.tilesN, p.M, sched, p.quantOut, p.quantScaleOut, static_cast<int32_t>(p.N / 2)};
         opapi::KernelTimer timer("gmm_requant", stream);
         hipLaunchKernelGGL(RequantKernel, dim3(static_cast<unsigned>(p.M)), dim3(256), 0, stream, ra);
         e = hipGetLastError();
