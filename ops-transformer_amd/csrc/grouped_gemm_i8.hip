@@ -16,11 +16,11 @@
 // XCD's L2); inside a group, bands of 4 m-tiles walk the n-tiles together so weight columns are reused from L2.
 //
 // Two kernels share the tile decode and the epilogue:
-//   StreamGemmKernel  the fast path (K-contiguous weights, K a multiple of 64).  Persistent workgroups; operands go
-//                     global -> LDS with global_load_lds_dwordx4 into a ring of 4..8 stages of 64 k-bytes, so several
+//   StreamGemmKernel  the fast path (K-contiguous weights, K a multiple of 128).  Persistent workgroups; operands go
+//                     global -> LDS with global_load_lds_dwordx4 into a ring of 3..8 stages of 128 (or 64) k-bytes, so several
 //                     stages of weights are in flight per CU with no staging registers, and the ring keeps filling
 //                     with the next tile's first steps while the current tile's epilogue runs.
-//   GenericGemmKernel byte-wise loader for row-major [K, N] weights and for K not a multiple of 64: correct, slow.
+//   GenericGemmKernel byte-wise loader for row-major [K, N] weights and for K not a multiple of 128: correct, slow.
 // LDS rows are XOR-swizzled in 16-byte chunks so that the 16 lanes the LDS serves per clock (64 banks) never collide,
 // for the DMA writes as well as for the MFMA operand reads.
 #include "grouped_gemm_i8.h"
@@ -28,6 +28,7 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "opapi_common.h"
@@ -37,6 +38,8 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float Float2 __attribute__((ext_vector_type(2)));
+typedef __bf16 Bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kTileN = 256;
 constexpr int kWavesN = 4;
@@ -128,7 +131,6 @@ struct KernelArgs {
     int32_t groups;
     int32_t tilesN;
     int32_t halfN;  // N / 2 (kSwiglu)
-    const int32_t* sched;
     void* out;
     int32_t outDtype;
     const void* scale;
@@ -149,13 +151,15 @@ struct TileInfo {
 };
 
 // Position `local` of the XCD share that starts at logical tile `xcdFirst`.
+// `sched` is passed to the kernels as a __restrict__ parameter of its own: nothing in a GEMM kernel writes the table,
+// and telling the compiler so keeps these wave-uniform lookups on the scalar unit even after the kernel's stores.
 template <int kTileM, bool kSwiglu>
-__device__ __forceinline__ TileInfo DecodeTile(const KernelArgs& a, int64_t xcdFirst, int64_t perXcd, int64_t totalTiles,
-                                               int64_t local) {
+__device__ __forceinline__ TileInfo DecodeTile(const KernelArgs& a, const int32_t* __restrict__ sched, int64_t xcdFirst,
+                                               int64_t perXcd, int64_t totalTiles, int64_t local) {
     TileInfo t{};
     const int64_t logical = xcdFirst + local;
     if (local >= perXcd || logical >= totalTiles) return t;
-    const int32_t* const rowStartTbl = a.sched + 2;
+    const int32_t* const rowStartTbl = sched + 2;
     const int32_t* const rowCountTbl = rowStartTbl + a.groups;
     const int32_t* const tilePrefix = rowCountTbl + a.groups;
     const int32_t q = static_cast<int32_t>(logical / a.tilesN);
@@ -204,37 +208,72 @@ __device__ __forceinline__ uint16_t ToBf16(float f) {
 
 // Epilogue of one tile.  acc[mi][ni][v] is C[row, col] with row = waveRow0 + 32*mi + 8*(v/4) + 4*lhi + (v%4); the wave
 // owns column blocks ni = 0, 1, lane l32 inside each (plain: 64*waveN + 32*ni; kSwiglu: S column 32*waveN and its partner).
-// ldsRowScale holds the tile's per-row scales.  Contains workgroup barriers: every wave must call it.
+// Only the first mySub accumulator tiles of the wave are real.  ldsRowScale holds the tile's per-row scales.
+// Contains workgroup barriers: every wave must call it.
 template <int kSubM, int kTileM, Epilogue kEpi>
-__device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo& t, v16i (&acc)[kSubM][2], int waveRow0,
-                                             int waveN, int l32, int lhi, int tid, const float* ldsRowScale,
-                                             float* ldsRowMax) {
+__device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo& t, v16i (&acc)[kSubM][2], int mySub,
+                                             int waveRow0, int waveN, int l32, int lhi, int tid,
+                                             const float* ldsRowScale, float* ldsRowMax) {
     const int32_t rows = t.rows, rowBase = t.rowBase, group = t.group;
     if (kEpi == Epilogue::kInt32 || kEpi == Epilogue::kDequant) {
         const bool hasRowScale = a.rowScale != nullptr;
+        const int32_t n0 = t.colBase + 64 * waveN + l32;  // column block 0; block 1 is 32 columns further
+        const bool valid0 = n0 < a.N, valid1 = n0 + 32 < a.N;
+        float sc0 = 0.0f, sc1 = 0.0f;
+        if (kEpi == Epilogue::kDequant) {
+            if (valid0) sc0 = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + n0, a.scaleDtype);
+            if (valid1) sc1 = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + n0 + 32, a.scaleDtype);
+        }
+        // 16-bit outputs: a lane holds one column of each block, i.e. 2-byte pieces 64 bytes apart.  Neighbouring lanes
+        // swap one value so that an even lane owns columns (c, c+1) of block 0 and the odd lane next to it the same pair
+        // of block 1; every lane then stores one aligned 32-bit word and a half-wave covers a whole 128-byte row segment.
+        const bool pairStores = kEpi == Epilogue::kDequant && a.outDtype != 0 && (a.N & 1) == 0 &&
+                                t.colBase + 64 * waveN + 64 <= a.N;  // wave-uniform
+        const bool oddLane = (l32 & 1) != 0;
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-            const int32_t n = t.colBase + 64 * waveN + 32 * ni + l32;
-            const bool nValid = n < a.N;
-            float sc = 0.0f;
-            if (kEpi == Epilogue::kDequant && nValid) sc = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + n, a.scaleDtype);
+        for (int mi = 0; mi < kSubM; ++mi) {
+            if (mi >= mySub || waveRow0 + 32 * mi >= rows) continue;
 #pragma unroll
-            for (int mi = 0; mi < kSubM; ++mi) {
-                if (waveRow0 + 32 * mi >= rows) continue;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int r = waveRow0 + 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
-                    if (r >= rows || !nValid) continue;
-                    const int64_t o = static_cast<int64_t>(rowBase + r) * a.N + n;
-                    if (kEpi == Epilogue::kInt32) {
-                        static_cast<int32_t*>(a.out)[o] = acc[mi][ni][v];
-                    } else {
-                        float y = __fmul_rn(static_cast<float>(acc[mi][ni][v]), sc);
-                        if (hasRowScale) y = __fmul_rn(y, ldsRowScale[r]);
-                        if (a.outDtype == 27) static_cast<uint16_t*>(a.out)[o] = ToBf16(y);
-                        else if (a.outDtype == 1) static_cast<__half*>(a.out)[o] = __float2half_rn(y);
-                        else static_cast<float*>(a.out)[o] = y;
-                    }
+            for (int v = 0; v < 16; ++v) {
+                const int r = waveRow0 + 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
+                const int64_t rowOff = static_cast<int64_t>(rowBase + r) * a.N;
+                if (kEpi == Epilogue::kInt32) {
+                    if (r < rows && valid0) static_cast<int32_t*>(a.out)[rowOff + n0] = acc[mi][0][v];
+                    if (r < rows && valid1) static_cast<int32_t*>(a.out)[rowOff + n0 + 32] = acc[mi][1][v];
+                    continue;
+                }
+                float y0 = __fmul_rn(static_cast<float>(acc[mi][0][v]), sc0);
+                float y1 = __fmul_rn(static_cast<float>(acc[mi][1][v]), sc1);
+                if (hasRowScale) {
+                    const float rs = ldsRowScale[r < rows ? r : 0];
+                    y0 = __fmul_rn(y0, rs);
+                    y1 = __fmul_rn(y1, rs);
+                }
+                if (a.outDtype == 0) {
+                    if (r < rows && valid0) static_cast<float*>(a.out)[rowOff + n0] = y0;
+                    if (r < rows && valid1) static_cast<float*>(a.out)[rowOff + n0 + 32] = y1;
+                    continue;
+                }
+                // both values rounded to nearest even and packed (low half = block 0)
+                uint32_t pk;
+                if (a.outDtype == 27) {
+                    const Float2 f = {y0, y1};
+                    pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));  // v_cvt_pk_bf16_f32
+                } else {
+                    pk = static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y0))) |
+                         (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y1))) << 16);
+                }
+                if (pairStores) {
+                    // quad_perm [1,0,3,2]: exchange with the lane whose index differs in bit 0, then keep
+                    // (own block-0 value, neighbour's block-0 value) on even lanes and
+                    // (neighbour's block-1 value, own block-1 value) on odd lanes
+                    const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
+                    const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
+                    const int32_t col = oddLane ? n0 + 31 : n0;  // odd lane l: block 1, columns 32 + (l - 1), 32 + l
+                    if (r < rows) *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(a.out) + rowOff + col) = word;
+                } else {
+                    if (r < rows && valid0) static_cast<uint16_t*>(a.out)[rowOff + n0] = static_cast<uint16_t>(pk & 0xffffu);
+                    if (r < rows && valid1) static_cast<uint16_t*>(a.out)[rowOff + n0 + 32] = static_cast<uint16_t>(pk >> 16);
                 }
             }
         }
@@ -248,6 +287,7 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
         }
 #pragma unroll
         for (int mi = 0; mi < kSubM; ++mi) {
+            if (mi >= mySub) continue;  // wave-uniform
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int r = waveRow0 + 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
@@ -257,7 +297,9 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                     const float xs = ldsRowScale[r];
                     const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), xs), scA);
                     const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xs), scB);
-                    s = __fmul_rn(__fdiv_rn(ca, __fadd_rn(1.0f, expf(-ca))), cb);
+                    // swish(ca) * cb with the hardware exp2 / reciprocal: a few ulp from the correctly rounded value,
+                    // far inside the +-1 LSB the int8 requantisation is held to
+                    s = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
                     a.sOut[static_cast<int64_t>(rowBase + r) * a.halfN + j] = s;
                 }
                 // max |S| of this row over the wave's 32 columns, kept by the first lane of each half-wave
@@ -279,27 +321,41 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
 }
 
 // ---------------------------------------------------------------------------------------------- fast path: LDS-DMA ring
-constexpr int kDmaStep = 64;  // k-bytes per ring stage
-
-template <int kSubM, int kWavesM>
+// kStep = k-bytes per ring stage: 128 streams weights in whole 128-byte lines (best HBM efficiency) when three such
+// stages fit in LDS, 64 allows a deeper ring for the tall tiles.
+// The tile's rows are split over one or two wave rows: wave row 0 owns kSub0 MFMA tiles (32 rows each), wave row 1 the
+// next kSub1 (kSub1 <= kSub0; kSub1 == 0 means four waves only).
+template <int kSub0, int kSub1, int kStep>
 struct StreamCfg {
+    static_assert(kSub1 <= kSub0, "wave row 0 is the taller one");
+    static constexpr int kWavesM = kSub1 > 0 ? 2 : 1;
     static constexpr int kWaves = kWavesN * kWavesM;
     static constexpr int kThreads = 64 * kWaves;
-    static constexpr int kTileM = 32 * kSubM * kWavesM;
-    static constexpr int kStageBytes = (kTileM + kTileN) * kDmaStep;
+    static constexpr int kTileM = 32 * (kSub0 + kSub1);
+    static constexpr int kStageBytes = (kTileM + kTileN) * kStep;
     static constexpr int kScratchBytes = (1 + kWavesN) * kTileM * 4;
     static constexpr int kStagesFit = (kLdsBudget - kScratchBytes) / kStageBytes;
     static constexpr int kStages = kStagesFit > 8 ? 8 : kStagesFit;
     static constexpr int kLdsBytes = kStages * kStageBytes + kScratchBytes;
-    // one DMA instruction moves 64 lanes x 16 bytes = 16 rows of 64 k-bytes
-    static constexpr int kInstrA = kTileM * kDmaStep / 1024;
-    static constexpr int kInstr = (kTileM + kTileN) * kDmaStep / 1024;
+    // one DMA instruction moves 64 lanes x 16 bytes = kRowsPerInstr tile rows of kStep k-bytes
+    static constexpr int kChunksPerRow = kStep / kChunk;
+    static constexpr int kRowsPerInstr = 64 / kChunksPerRow;
+    static constexpr int kInstrA = kTileM / kRowsPerInstr;
+    static constexpr int kInstr = (kTileM + kTileN) / kRowsPerInstr;
+    static_assert(kTileM % kRowsPerInstr == 0, "tile rows must fill whole DMA instructions");
     static constexpr int kMaxPerWave = (kInstr + kWaves - 1) / kWaves;
-    static_assert(kStages >= 3, "the ring needs at least three stages");
+    static_assert(kStages >= 2, "the ring needs at least two stages");
     static_assert((kStages - 2) * kMaxPerWave <= 63, "vmcnt is a 6-bit counter");
 };
 
-__device__ __forceinline__ int Lds64Offset(int row, int chunk) { return row * kDmaStep + ((chunk ^ ((row >> 2) & 3)) << 4); }
+// Byte offset of 16-byte chunk `chunk` of row `row` in a stage whose rows are kStep bytes.  The LDS serves 16 lanes per
+// clock out of 64 banks (256 bytes): the chunk index is XOR-ed with row bits such that 16 consecutive rows reading the
+// same logical chunk land in 16 different 16-byte bank groups.
+template <int kStep>
+__device__ __forceinline__ int LdsOffset(int row, int chunk) {
+    if (kStep == 64) return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4);
+    return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4);
+}
 
 // 16 bytes per lane from (uniform base + 32-bit lane offset) straight into LDS at ldsDst + lane * 16.  The compiler does
 // not see this as a memory instruction: completion is awaited with WaitVmcnt below.
@@ -324,9 +380,11 @@ __device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leavi
 
 // Persistent: the grid is one workgroup per CU (a multiple of 8); workgroup b serves XCD b % 8 and walks that XCD's
 // share of the tile list with stride gridDim / 8.
-template <int kSubM, int kWavesM, Epilogue kEpi>
-__global__ __launch_bounds__(256 * kWavesM) void StreamGemmKernel(KernelArgs a) {
-    using Cfg = StreamCfg<kSubM, kWavesM>;
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi>
+__global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
+    KernelArgs a, const int32_t* __restrict__ sched) {
+    using Cfg = StreamCfg<kSub0, kSub1, kStep>;
+    constexpr int kSubM = kSub0;  // accumulator tiles per wave (wave row 1 uses the first kSub1 of them)
     constexpr int kTileM = Cfg::kTileM;
     constexpr int kStages = Cfg::kStages;
     constexpr int kStageBytes = Cfg::kStageBytes;
@@ -343,16 +401,16 @@ __global__ __launch_bounds__(256 * kWavesM) void StreamGemmKernel(KernelArgs a) 
     const int l32 = lane & 31;
     const int lhi = lane >> 5;
 
-    const int64_t totalTiles = static_cast<int64_t>(a.sched[1]) * a.tilesN;
+    const int64_t totalTiles = static_cast<int64_t>(sched[1]) * a.tilesN;
     const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
     const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
     const int64_t slots = gridDim.x / kXcds;
-    auto decode = [&](int64_t local) { return DecodeTile<kTileM, kSwiglu>(a, xcdFirst, perXcd, totalTiles, local); };
+    auto decode = [&](int64_t local) { return DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, local); };
 
     int64_t local = blockIdx.x / kXcds;
     TileInfo cur = decode(local);
     if (!cur.valid) return;
-    const int kSteps = a.K / kDmaStep;
+    const int kSteps = a.K / kStep;
 
     // ---- issue side: runs kStages - 1 steps ahead of the compute side, across tile boundaries ----
     TileInfo iss = cur;
@@ -368,26 +426,30 @@ __global__ __launch_bounds__(256 * kWavesM) void StreamGemmKernel(KernelArgs a) 
     auto setupIssue = [&]() {
         issX = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(iss.rowBase) * a.K;
         issW = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(iss.group) * a.wGroupStride;
-        const int rowLimit = a.M - 1 - iss.rowBase;  // rows past the tile read whatever follows in x, never beyond it
-        const int rowIn = lane >> 2;
-        const int slot = lane & 3;
+        // lane -> (row inside the instruction, LDS chunk slot); the global chunk it fetches is the one LdsOffset puts there
+        const int rowIn = lane / Cfg::kChunksPerRow;
+        const int slot = lane % Cfg::kChunksPerRow;
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
             const int j = wave + q * Cfg::kWaves;
             if (j < Cfg::kInstrA) {
-                const int r = 16 * j + rowIn;
-                const int c = slot ^ ((r >> 2) & 3);
-                laneOff[q] = static_cast<uint32_t>(min(r, rowLimit) * a.K + c * kChunk);
+                // rows past the tile's last row are never used: such lanes re-read the last real row (same cache
+                // lines as its own lanes), and an instruction wholly past it reads one chunk, so the number of DMAs
+                // per stage stays constant while the activation traffic follows the real row count
+                const int r = Cfg::kRowsPerInstr * j + rowIn;
+                const int c = (LdsOffset<kStep>(r, slot) >> 4) % Cfg::kChunksPerRow;
+                const bool wholeInstrPast = Cfg::kRowsPerInstr * j >= iss.rows;
+                laneOff[q] = wholeInstrPast ? 0u : static_cast<uint32_t>(min(r, iss.rows - 1) * a.K + c * kChunk);
             } else {
-                const int r = 16 * (j - Cfg::kInstrA) + rowIn;
-                const int c = slot ^ ((r >> 2) & 3);
+                const int r = Cfg::kRowsPerInstr * (j - Cfg::kInstrA) + rowIn;
+                const int c = (LdsOffset<kStep>(r, slot) >> 4) % Cfg::kChunksPerRow;
                 laneOff[q] = static_cast<uint32_t>(ChannelOfRow<kSwiglu>(a, iss, r) * a.K + c * kChunk);
             }
         }
     };
     auto issueStage = [&](int ring) {
         char* const dst = lds + ring * kStageBytes;
-        const int kOff = issStep * kDmaStep;
+        const int kOff = issStep * kStep;
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
             const int j = wave + q * Cfg::kWaves;
@@ -415,7 +477,8 @@ __global__ __launch_bounds__(256 * kWavesM) void StreamGemmKernel(KernelArgs a) 
         ldsRowScale[tid] = a.rowScale[cur.rowBase + (tid < cur.rows ? tid : cur.rows - 1)];
     }
 
-    const int waveRow0 = waveM * 32 * kSubM;
+    const int waveRow0 = waveM * 32 * kSub0;
+    const int mySub = waveM == 0 ? kSub0 : kSub1;  // MFMA tiles of this wave
     const int bRow0 = kSwiglu ? 32 * waveN : 64 * waveN;
     const int bRowStep = kSwiglu ? kTileN / 2 : 32;
     v16i acc[kSubM][2];
@@ -442,23 +505,25 @@ __global__ __launch_bounds__(256 * kWavesM) void StreamGemmKernel(KernelArgs a) 
             __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
             issueStage(ring == 0 ? kStages - 1 : ring - 1);
             const char* const A = lds + ring * kStageBytes;
-            const char* const B = A + kTileM * kDmaStep;
+            const char* const B = A + kTileM * kStep;
 #pragma unroll
-            for (int ks = 0; ks < kDmaStep / 32; ++ks) {
+            for (int ks = 0; ks < kStep / 32; ++ks) {
                 const int chunk = 2 * ks + lhi;
-                const v4i b0 = *reinterpret_cast<const v4i*>(B + Lds64Offset(bRow0 + l32, chunk));
-                const v4i b1 = *reinterpret_cast<const v4i*>(B + Lds64Offset(bRow0 + bRowStep + l32, chunk));
+                const v4i b0 = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + l32, chunk));
+                const v4i b1 = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + bRowStep + l32, chunk));
 #pragma unroll
                 for (int mi = 0; mi < kSubM; ++mi) {
-                    const v4i av = *reinterpret_cast<const v4i*>(A + Lds64Offset(waveRow0 + mi * 32 + l32, chunk));
-                    acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b0, acc[mi][0], 0, 0, 0);
-                    acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, acc[mi][1], 0, 0, 0);
+                    if (mi < kSub1 || waveM == 0) {  // compile-time true for the tiles both wave rows have
+                        const v4i av = *reinterpret_cast<const v4i*>(A + LdsOffset<kStep>(waveRow0 + mi * 32 + l32, chunk));
+                        acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b0, acc[mi][0], 0, 0, 0);
+                        acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, acc[mi][1], 0, 0, 0);
+                    }
                 }
             }
             ring = ring + 1 == kStages ? 0 : ring + 1;
         }
 
-        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, waveRow0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
+        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
         // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
         // stores and the DMAs in flight, which had the whole epilogue to land) before counting DMAs again.
         WaitVmcnt<0>();
@@ -478,7 +543,7 @@ __device__ __forceinline__ int Lds128Offset(int row, int chunk) { return row * k
 // One tile per workgroup (grid = static upper bound of tiles), 4 waves, operands gathered byte by byte through
 // registers into a single LDS buffer.  Handles any K and both weight layouts.
 template <int kSubM, Epilogue kEpi>
-__global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a) {
+__global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a, const int32_t* __restrict__ sched) {
     constexpr int kThreads = 256;
     constexpr int kTileM = 32 * kSubM;
     constexpr int kChunksPerRow = kGenStep / kChunk;
@@ -496,10 +561,10 @@ __global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a) {
     const int l32 = lane & 31;
     const int lhi = lane >> 5;
 
-    const int64_t totalTiles = static_cast<int64_t>(a.sched[1]) * a.tilesN;
+    const int64_t totalTiles = static_cast<int64_t>(sched[1]) * a.tilesN;
     const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
     const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
-    const TileInfo t = DecodeTile<kTileM, kSwiglu>(a, xcdFirst, perXcd, totalTiles, blockIdx.x / kXcds);
+    const TileInfo t = DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, blockIdx.x / kXcds);
     if (!t.valid) return;
     if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
         ldsRowScale[tid] = a.rowScale[t.rowBase + (tid < t.rows ? tid : t.rows - 1)];
@@ -559,7 +624,7 @@ __global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a) {
         }
         __syncthreads();
     }
-    TileEpilogue<kSubM, kTileM, kEpi>(a, t, acc, 0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
+    TileEpilogue<kSubM, kTileM, kEpi>(a, t, acc, kSubM, 0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
 }
 
 // ---------------------------------------------------------------------------------------------- requantisation
@@ -625,10 +690,10 @@ int DeviceCuCount() {
     return count;
 }
 
-template <int kSubM, int kWavesM, Epilogue kEpi>
-hipError_t LaunchStream(const KernelArgs& args, int64_t maxTiles, hipStream_t stream) {
-    using Cfg = StreamCfg<kSubM, kWavesM>;
-    auto kernel = StreamGemmKernel<kSubM, kWavesM, kEpi>;
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi>
+hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
+    using Cfg = StreamCfg<kSub0, kSub1, kStep>;
+    auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
     if (attr != hipSuccess) return attr;
@@ -637,33 +702,37 @@ hipError_t LaunchStream(const KernelArgs& args, int64_t maxTiles, hipStream_t st
     if (grid > maxTiles) grid = maxTiles;
     grid = grid / kXcds * kXcds;
     if (grid < kXcds) grid = kXcds;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, args);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, args, sched);
     return hipGetLastError();
 }
 
+// Tile heights and their (wave row 0, wave row 1, k-step) shapes.  128-byte steps with a ring of three or more stages
+// stream best; 192 and 256 rows only leave room for two such stages.
 template <Epilogue kEpi>
-hipError_t LaunchStreamShape(const Plan& plan, const KernelArgs& args, hipStream_t stream) {
+hipError_t LaunchStreamShape(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
     switch (plan.tileM) {
-        case 32: return LaunchStream<1, 1, kEpi>(args, plan.maxTiles, stream);
-        case 64: return LaunchStream<1, 2, kEpi>(args, plan.maxTiles, stream);
-        case 128: return LaunchStream<2, 2, kEpi>(args, plan.maxTiles, stream);
-        case 192: return LaunchStream<3, 2, kEpi>(args, plan.maxTiles, stream);
-        default: return LaunchStream<4, 2, kEpi>(args, plan.maxTiles, stream);
+        case 32: return LaunchStream<1, 0, 128, kEpi>(args, sched, plan.maxTiles, stream);
+        case 64: return LaunchStream<1, 1, 128, kEpi>(args, sched, plan.maxTiles, stream);
+        case 96: return LaunchStream<2, 1, 128, kEpi>(args, sched, plan.maxTiles, stream);
+        case 128: return LaunchStream<2, 2, 128, kEpi>(args, sched, plan.maxTiles, stream);
+        case 160: return LaunchStream<3, 2, 128, kEpi>(args, sched, plan.maxTiles, stream);
+        case 192: return LaunchStream<3, 3, 128, kEpi>(args, sched, plan.maxTiles, stream);
+        default: return LaunchStream<4, 4, 128, kEpi>(args, sched, plan.maxTiles, stream);
     }
 }
 
 template <Epilogue kEpi>
-hipError_t LaunchGenericShape(const Plan& plan, const KernelArgs& args, hipStream_t stream) {
+hipError_t LaunchGenericShape(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
     const dim3 grid(static_cast<unsigned>(plan.maxTiles));
-    if (plan.tileM <= 32) hipLaunchKernelGGL((GenericGemmKernel<1, kEpi>), grid, dim3(256), 0, stream, args);
-    else hipLaunchKernelGGL((GenericGemmKernel<4, kEpi>), grid, dim3(256), 0, stream, args);
+    if (plan.tileM <= 32) hipLaunchKernelGGL((GenericGemmKernel<1, kEpi>), grid, dim3(256), 0, stream, args, sched);
+    else hipLaunchKernelGGL((GenericGemmKernel<4, kEpi>), grid, dim3(256), 0, stream, args, sched);
     return hipGetLastError();
 }
 
-// The DMA ring needs K-contiguous weights, whole 64-byte k steps, 16-byte aligned bases and 32-bit offsets inside one
+// The DMA ring needs K-contiguous weights, whole 128-byte k steps, 16-byte aligned bases and 32-bit offsets inside one
 // expert's weights.
 bool StreamOk(const Problem& p) {
-    return p.wKMajor && p.K % kDmaStep == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
+    return p.wKMajor && p.K % 128 == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
            reinterpret_cast<uintptr_t>(p.w) % kChunk == 0 && p.N * p.K < (1ll << 31);
 }
 
@@ -674,18 +743,27 @@ uint64_t Align256(uint64_t v) { return (v + 255) / 256 * 256; }
 Plan MakePlan(const Problem& p) {
     Plan plan;
     const int64_t groups = p.groups > 0 ? p.groups : 1;
-    const double want = static_cast<double>(p.M) / static_cast<double>(groups) * 1.3;
+    // tile height: the mean group size plus a quarter, so that almost every group is covered by one m-tile and its
+    // weights are streamed exactly once
+    const double want = static_cast<double>(p.M) / static_cast<double>(groups) * 1.25;
     if (StreamOk(p)) {
-        static const int kShapes[] = {32, 64, 128, 192, 256};
+        static const int kShapes[] = {32, 64, 96, 128, 160, 192, 256};
         plan.tileM = 256;
         for (int s : kShapes) {
             if (static_cast<double>(s) >= want) { plan.tileM = s; break; }
+        }
+        // tuning override: OPAPI_GEMM_TILE_M=<one of the shapes above>
+        if (const char* env = std::getenv("OPAPI_GEMM_TILE_M")) {
+            const int forced = std::atoi(env);
+            for (int s : kShapes) {
+                if (s == forced) plan.tileM = s;
+            }
         }
     } else {
         plan.tileM = want <= 32.0 ? 32 : 128;
     }
     plan.wavesM = plan.tileM >= 64 && StreamOk(p) ? 2 : 1;
-    plan.subTilesM = plan.tileM / 32 / plan.wavesM;
+    plan.subTilesM = (plan.tileM / 32 + plan.wavesM - 1) / plan.wavesM;
     const int64_t cols = p.epilogue == Epilogue::kSwiglu ? p.N / 2 : p.N;
     const int64_t colsPerTile = p.epilogue == Epilogue::kSwiglu ? kTileN / 2 : kTileN;
     plan.tilesN = static_cast<int32_t>((cols + colsPerTile - 1) / colsPerTile);
@@ -739,7 +817,6 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.groups = p.groups;
     ka.tilesN = plan.tilesN;
     ka.halfN = static_cast<int32_t>(p.N / 2);
-    ka.sched = sched;
     ka.out = p.out;
     ka.outDtype = p.outDtype;
     ka.scale = p.scale;
@@ -755,16 +832,16 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
                                  : p.epilogue == Epilogue::kDequant ? "gmm_dequant" : "gmm_int32", stream);
         switch (p.epilogue) {
             case Epilogue::kInt32:
-                e = fast ? LaunchStreamShape<Epilogue::kInt32>(plan, ka, stream)
-                         : LaunchGenericShape<Epilogue::kInt32>(plan, ka, stream);
+                e = fast ? LaunchStreamShape<Epilogue::kInt32>(plan, ka, sched, stream)
+                         : LaunchGenericShape<Epilogue::kInt32>(plan, ka, sched, stream);
                 break;
             case Epilogue::kDequant:
-                e = fast ? LaunchStreamShape<Epilogue::kDequant>(plan, ka, stream)
-                         : LaunchGenericShape<Epilogue::kDequant>(plan, ka, stream);
+                e = fast ? LaunchStreamShape<Epilogue::kDequant>(plan, ka, sched, stream)
+                         : LaunchGenericShape<Epilogue::kDequant>(plan, ka, sched, stream);
                 break;
             case Epilogue::kSwiglu:
-                e = fast ? LaunchStreamShape<Epilogue::kSwiglu>(plan, ka, stream)
-                         : LaunchGenericShape<Epilogue::kSwiglu>(plan, ka, stream);
+                e = fast ? LaunchStreamShape<Epilogue::kSwiglu>(plan, ka, sched, stream)
+                         : LaunchGenericShape<Epilogue::kSwiglu>(plan, ka, sched, stream);
                 break;
         }
         if (e != hipSuccess) return e;
