@@ -503,7 +503,6 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             if (dmaPerStage == Cfg::kMaxPerWave) WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
             else WaitVmcnt<(kStages - 2) * (Cfg::kMaxPerWave - 1)>();
             __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
-            issueStage(ring == 0 ? kStages - 1 : ring - 1);
             const char* const A = lds + ring * kStageBytes;
             const char* const B = A + kTileM * kStep;
 #pragma unroll
@@ -519,6 +518,9 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                         acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, acc[mi][1], 0, 0, 0);
                     }
                 }
+                // The refill of the stage freed by the barrier is issued behind the first block of MFMAs: its scalar
+                // address work then runs in the shadow of the matrix pipe instead of in front of it.
+                if (ks == 0) issueStage(ring == 0 ? kStages - 1 : ring - 1);
             }
             ring = ring + 1 == kStages ? 0 : ring + 1;
         }

@@ -100,44 +100,71 @@ struct CountOutputs {
     int32_t expertNum;
 };
 
-// One workgroup of 1024 threads; each thread owns bins/1024 (1 or 2) digit values.
+// One workgroup of 1024 threads.  With B bins, 1024 / B threads share each digit value (one thread owns two values when
+// B = 2048): the slices are cut into that many segments, every thread totals its segment, the segment totals are
+// prefixed through LDS, and a second walk turns the table into exclusive offsets.
 __global__ __launch_bounds__(1024) void DigitScanKernel(SortPass p, CountOutputs co) {
+    __shared__ int32_t segTotal[2048];  // [segment][bin]
     __shared__ int32_t partial[1024];
     const int bins = 1 << p.bits;
-    const int perThread = (bins + 1023) / 1024;
-    int32_t totals[2] = {0, 0};
-    for (int j = 0; j < perThread; ++j) {
-        const int b = threadIdx.x * perThread + j;
-        if (b >= bins) break;
+    const int binsPerThread = bins > 1024 ? bins / 1024 : 1;
+    const int segs = bins >= 1024 ? 1 : 1024 / bins;
+    const int seg = bins >= 1024 ? 0 : threadIdx.x / bins;
+    const int bin0 = bins >= 1024 ? threadIdx.x * binsPerThread : threadIdx.x % bins;
+    const int slicesPerSeg = (p.numSlices + segs - 1) / segs;
+    const int sBegin = seg * slicesPerSeg;
+    const int sEnd = min(p.numSlices, sBegin + slicesPerSeg);
+    for (int j = 0; j < binsPerThread; ++j) {
+        const int b = bin0 + j;
         int32_t run = 0;
-        for (int s = 0; s < p.numSlices; ++s) {
-            const int32_t v = p.table[static_cast<int64_t>(s) * bins + b];
-            p.table[static_cast<int64_t>(s) * bins + b] = run;
-            run += v;
-        }
-        totals[j] = run;
+#pragma unroll 8
+        for (int s = sBegin; s < sEnd; ++s) run += p.table[static_cast<int64_t>(s) * bins + b];
+        segTotal[seg * bins + b] = run;
     }
-    const int32_t mine = totals[0] + totals[1];
+    __syncthreads();
+    // per digit value: offset of this thread's segment inside the value, and the value's total
+    int32_t segBase[2] = {0, 0}, total[2] = {0, 0};
+    for (int j = 0; j < binsPerThread; ++j) {
+        const int b = bin0 + j;
+        for (int g = 0; g < segs; ++g) {
+            const int32_t v = segTotal[g * bins + b];
+            if (g < seg) segBase[j] += v;
+            total[j] += v;
+        }
+    }
+    // exclusive scan of the totals across digit values (threads of segment 0 carry them, the others contribute 0)
+    const int32_t mine = seg == 0 ? total[0] + total[1] : 0;
     partial[threadIdx.x] = mine;
     __syncthreads();
-    // Hillis-Steele inclusive scan over the 1024 per-thread sums
     for (int d = 1; d < 1024; d <<= 1) {
         const int32_t add = threadIdx.x >= d ? partial[threadIdx.x - d] : 0;
         __syncthreads();
         partial[threadIdx.x] += add;
         __syncthreads();
     }
-    int32_t base = partial[threadIdx.x] - mine;
-    for (int j = 0; j < perThread; ++j) {
-        const int b = threadIdx.x * perThread + j;
-        if (b >= bins) break;
-        p.binBase[b] = base;
-        p.binTotal[b] = totals[j];
-        if (b < co.expertNum) {
-            if (co.countOrCumsum != nullptr) co.countOrCumsum[b] = co.flag == 1 ? base + totals[j] : totals[j];
-            if (co.beforeCapacity != nullptr) co.beforeCapacity[b] = totals[j];
+    if (seg == 0) {
+        int32_t base = partial[threadIdx.x] - mine;
+        for (int j = 0; j < binsPerThread; ++j) {
+            const int b = bin0 + j;
+            p.binBase[b] = base;
+            p.binTotal[b] = total[j];
+            if (b < co.expertNum) {
+                if (co.countOrCumsum != nullptr) co.countOrCumsum[b] = co.flag == 1 ? base + total[j] : total[j];
+                if (co.beforeCapacity != nullptr) co.beforeCapacity[b] = total[j];
+            }
+            base += total[j];
         }
-        base += totals[j];
+    }
+    // second walk: table[slice][bin] becomes the number of keys with this digit in earlier slices
+    for (int j = 0; j < binsPerThread; ++j) {
+        const int b = bin0 + j;
+        int32_t run = segBase[j];
+#pragma unroll 4
+        for (int s = sBegin; s < sEnd; ++s) {
+            const int32_t v = p.table[static_cast<int64_t>(s) * bins + b];
+            p.table[static_cast<int64_t>(s) * bins + b] = run;
+            run += v;
+        }
     }
 }
 
