@@ -1,0 +1,286 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol the headers declare, and its first-phase entry points
+apply the reference's argument rules with the reference's return codes (the phase never touches device memory, so fake
+device pointers suffice).  Negative cases mirror the reference's own op_api / tiling unit tests:
+  moe/moe_init_routing_v2/tests/utest/ts_moe_init_routing_v2_tc.cpp:59-141
+  gmm/grouped_matmul_swiglu_quant/tests/ut/op_host/op_api/test_aclnn_grouped_matmul_swiglu_quant.cpp:38-63
+  gmm/grouped_matmul/tests/utest_aclnn/ts_aclnn_grouped_matmul.cpp
+  moe/moe_finalize_routing_v2/tests/ut/op_host/test_moe_finalize_routing_v2_tiling.cpp
+"""
+import ctypes
+import glob
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+NULLPTR, INVALID = 161001, 161002
+
+
+def _declared_symbols():
+    names = set()
+    for path in glob.glob(os.path.join(ROOT, "include", "**", "*.h"), recursive=True):
+        text = open(path).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        for m in re.finditer(r"(?:ACL_API|ACLNN_API|__attribute__\(\(visibility\(\"default\"\)\)\))\s+[\w\s\*]+?\b(\w+)\s*\(", text):
+            names.add(m.group(1))
+    return sorted(names)
+
+
+def test_headers_declare_the_expected_entry_points():
+    names = _declared_symbols()
+    for required in ["aclnnMoeInitRoutingV2GetWorkspaceSize", "aclnnMoeInitRoutingV2",
+                     "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize", "aclnnGroupedMatmulSwigluQuant",
+                     "aclnnGroupedMatmulV4GetWorkspaceSize", "aclnnGroupedMatmulV4",
+                     "aclnnMoeFinalizeRoutingV2GetWorkspaceSize", "aclnnMoeFinalizeRoutingV2",
+                     "aclCreateTensor", "aclDestroyTensor", "aclCreateTensorList", "aclDestroyTensorList", "aclrtMalloc",
+                     "aclrtMemcpy", "aclGetRecentErrMsg", "ResetCacheThreadLocal", "opapiKernelTimerEnable",
+                     "opapiKernelTimerReport"]:
+        assert required in names, required
+
+
+def test_library_exports_every_declared_symbol(aclnn):
+    lib = ctypes.CDLL(aclnn.library_path())
+    missing = [n for n in _declared_symbols() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+# ------------------------------------------------------------------------------------------------ helpers
+F32, F16, I8, I32, I64, BF16 = 0, 1, 2, 3, 9, 27
+
+
+class T:
+    """Descriptor over a fake device address (phase 1 never dereferences it)."""
+    _next = 0x10000
+
+    def __init__(self, aclnn, shape, dtype, strides=None, data=True, fmt=2):
+        T._next += 0x10000
+        self.h = aclnn.create_tensor(list(shape), dtype, T._next if data else 0, strides, 0, fmt)
+
+
+def _status(aclnn, api, args):
+    try:
+        return 0, aclnn.workspace_size(api, args)
+    except aclnn.AclnnError as e:
+        assert e.message, "an error status must come with a message"
+        return e.code, e.message
+
+
+def _tl(aclnn, tensors):
+    arr = (ctypes.c_void_p * len(tensors))(*[t.h for t in tensors])
+    return aclnn.lib().aclCreateTensorList(arr, len(tensors))
+
+
+# ------------------------------------------------------------------------------------------------ routing
+def _routing_args(aclnn, T_=8, K=2, H=16, E=4, mode=0, C=0, flag=0, before=False, active=0, x_dtype=F32, **over):
+    x = T(aclnn, (T_, H), x_dtype)
+    idx = T(aclnn, (T_, K), I32)
+    if mode == 0:
+        rows = T_ * K if active == 0 else min(T_ * K, active)
+        ex = T(aclnn, over.get("ex_shape", (rows, H)), x_dtype)
+    else:
+        ex = T(aclnn, over.get("ex_shape", (E, C, H)), x_dtype)
+    ri = T(aclnn, over.get("ri_shape", (T_ * K,)), I32)
+    cnt = T(aclnn, over.get("cnt_shape", (E,)), I32) if over.get("with_cnt", flag > 0) else None
+    bef = T(aclnn, (E,), I32) if before else None
+    return [x.h, idx.h, active, C, E, mode, flag, before, ex.h, ri.h, cnt.h if cnt else None, bef.h if bef else None]
+
+
+def test_routing_valid_shapes(aclnn):
+    for kw in [dict(), dict(flag=1), dict(flag=2), dict(mode=1, C=3, before=True), dict(active=5), dict(x_dtype=I8),
+               dict(x_dtype=BF16, flag=1), dict(T_=0)]:
+        code, ws = _status(aclnn, "aclnnMoeInitRoutingV2", _routing_args(aclnn, **kw))
+        assert code == 0, (kw, ws)
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    (dict(mode=2), "dropPadMode should be 0 or 1"),
+    (dict(flag=3), "should be 0, 1 or 2"),
+    (dict(flag=1, E=0, with_cnt=False), "expertNum should be greater than 0"),
+    (dict(mode=1, C=0), "greater than 0 when dropPadMode is 1"),
+    (dict(mode=1, C=9, T_=8), "cannot be less than expertCapacity"),
+    (dict(ex_shape=(15, 16)), "first dim of expandedX"),
+    (dict(ex_shape=(16, 17)), "second dim of expandedX"),
+    (dict(ri_shape=(15,)), "first dim of expandedRowIdx"),
+    (dict(flag=1, cnt_shape=(5,)), "expertTokensCountOrCumsum"),
+    (dict(active=-1), "activeNum cannot be less than 0"),
+    (dict(E=-1), "expertNum cannot be less than 0"),
+])
+def test_routing_invalid_arguments(aclnn, kw, fragment):
+    code, msg = _status(aclnn, "aclnnMoeInitRoutingV2", _routing_args(aclnn, **kw))
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_routing_null_and_rank_checks(aclnn):
+    args = _routing_args(aclnn)
+    args[0] = None
+    assert _status(aclnn, "aclnnMoeInitRoutingV2", args)[0] == NULLPTR
+    args = _routing_args(aclnn, flag=1, with_cnt=False)
+    assert _status(aclnn, "aclnnMoeInitRoutingV2", args)[0] == NULLPTR  # count output requested but absent
+    x3 = T(aclnn, (2, 2, 2), F32)
+    args = _routing_args(aclnn)
+    args[0] = x3.h
+    code, msg = _status(aclnn, "aclnnMoeInitRoutingV2", args)
+    assert code == INVALID and "dim number of x should be 2" in msg
+
+
+# ------------------------------------------------------------------------------------------------ SwiGLU quant
+def _swiglu_args(aclnn, M=192, K=2048, N=2048, E=4, **over):
+    x = T(aclnn, over.get("x_shape", (M, K)), over.get("x_dtype", I8))
+    w = T(aclnn, over.get("w_shape", (E, K, N)), over.get("w_dtype", I8), over.get("w_strides"), fmt=over.get("w_fmt", 2))
+    ws = T(aclnn, over.get("ws_shape", (E, N)), over.get("ws_dtype", F32))
+    xs = T(aclnn, over.get("xs_shape", (M,)), F32)
+    gl = T(aclnn, (over.get("gl_len", E),), over.get("gl_dtype", I64))
+    out = T(aclnn, over.get("out_shape", (M, N // 2)), I8)
+    outs = T(aclnn, (M,), F32)
+    return [x.h, w.h, None, None, ws.h, xs.h, gl.h, out.h, outs.h, None]
+
+
+def test_swiglu_valid(aclnn):
+    # shape of the reference op_api unit test, plus the widenings of this build
+    for kw in [dict(), dict(ws_dtype=BF16), dict(ws_dtype=F16), dict(gl_dtype=I32), dict(N=28672, K=4096, M=64, E=2),
+               dict(w_strides=[2048 * 2048, 1, 2048]), dict(gl_len=3)]:
+        code, ws = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, **kw))
+        assert code == 0, (kw, ws)
+    code, ws = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=16, K=256, N=512, E=4))
+    assert code == 0 and ws >= 16 * 256 * 4  # S workspace [M, N/2] fp32 plus tables
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    (dict(x_dtype=F16), "A8W8"),
+    (dict(w_fmt=29), "FRACTAL_NZ"),
+    (dict(N=2047, out_shape=(192, 1023), ws_shape=(4, 2047)), "must even number"),
+    (dict(ws_shape=(4, 2046)), "weightScale must be"),
+    (dict(xs_shape=(191,)), "xScale must be"),
+    (dict(out_shape=(192, 2048)), "output must be"),
+    (dict(gl_len=5), "Length of 'groupList' out of range"),
+    (dict(K=65536, w_shape=(4, 65536, 2048)), "need lower than"),
+    (dict(w_shape=(4, 1024, 2048)), "does not match x"),
+    (dict(w_strides=[2048 * 2048, 4096, 2]), "contiguous"),
+])
+def test_swiglu_invalid(aclnn, kw, fragment):
+    code, msg = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, **kw))
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_swiglu_null_and_empty(aclnn):
+    args = _swiglu_args(aclnn)
+    args[4] = None
+    assert _status(aclnn, "aclnnGroupedMatmulSwigluQuant", args)[0] == NULLPTR
+    # an empty groupList is a successful no-op with no workspace
+    code, ws = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, gl_len=0))
+    assert code == 0 and ws == 0
+
+
+# ------------------------------------------------------------------------------------------------ grouped matmul V4
+def _gmm_args(aclnn, M=64, K=256, N=128, E=4, scale_dtype=F32, out_dtype=BF16, per_token=True, **over):
+    x = _tl(aclnn, [T(aclnn, (M, K), over.get("x_dtype", I8))])
+    w = _tl(aclnn, [T(aclnn, over.get("w_shape", (E, K, N)), I8)])
+    scale = _tl(aclnn, [T(aclnn, (E, N), scale_dtype)]) if scale_dtype is not None else None
+    pt = _tl(aclnn, [T(aclnn, over.get("pt_shape", (M,)), F32)]) if per_token else None
+    gl = T(aclnn, (over.get("gl_len", E),), over.get("gl_dtype", I64))
+    out = _tl(aclnn, [T(aclnn, over.get("out_shape", (M, N)), out_dtype)])
+    args = [x, w, over.get("bias"), scale, over.get("offset"), None, None, pt, gl.h if over.get("with_gl", True) else None,
+            over.get("act_in"), None, None, over.get("split_item", 3), over.get("group_type", 0),
+            over.get("group_list_type", 0), over.get("act_type", 0), out, None, None]
+    return args
+
+
+def test_gmm_valid(aclnn):
+    for kw in [dict(), dict(scale_dtype=BF16), dict(out_dtype=F16), dict(scale_dtype=None, out_dtype=I32, per_token=False),
+               dict(group_list_type=1), dict(split_item=2), dict(gl_dtype=I32), dict(per_token=False)]:
+        code, ws = _status(aclnn, "aclnnGroupedMatmulV4", _gmm_args(aclnn, **kw))
+        assert code == 0, (kw, ws)
+
+
+def test_gmm_empty_optional_means_absent(aclnn):
+    # a shape-[0] per-token scale inside a list is "absent" (the reference's graph bridge passes it that way)
+    args = _gmm_args(aclnn, per_token=False)
+    args[7] = _tl(aclnn, [T(aclnn, (0,), F32)])
+    assert _status(aclnn, "aclnnGroupedMatmulV4", args)[0] == 0
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    (dict(x_dtype=F16), "INT8"),
+    (dict(scale_dtype=BF16, out_dtype=F16), "scale/output dtype pair"),
+    (dict(scale_dtype=None, out_dtype=BF16, per_token=False), "must be INT32"),
+    (dict(group_type=2), "groupType 0"),
+    (dict(split_item=0), "splitItem 2 or 3"),
+    (dict(group_list_type=2), "sparse"),
+    (dict(group_list_type=3), "groupListType"),
+    (dict(act_type=3), "GELU_ERR_FUNC"),
+    (dict(act_type=1), "actType 1"),
+    (dict(gl_len=3), "should be equal to weight dim 0"),
+    (dict(pt_shape=(63,)), "perTokenScale must be"),
+    (dict(out_shape=(64, 127)), "y must be"),
+    (dict(with_gl=False), "groupListOptional(tensor) is required"),
+])
+def test_gmm_invalid(aclnn, kw, fragment):
+    code, msg = _status(aclnn, "aclnnGroupedMatmulV4", _gmm_args(aclnn, **kw))
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_gmm_reserved_arguments_and_nulls(aclnn):
+    args = _gmm_args(aclnn)
+    args[9] = _tl(aclnn, [T(aclnn, (4,), F32)])
+    code, msg = _status(aclnn, "aclnnGroupedMatmulV4", args)
+    assert code == INVALID and "activationInputOptional must be nullptr" in msg
+    args = _gmm_args(aclnn)
+    args[0] = None
+    assert _status(aclnn, "aclnnGroupedMatmulV4", args)[0] == NULLPTR
+    args = _gmm_args(aclnn)
+    args[16] = None
+    assert _status(aclnn, "aclnnGroupedMatmulV4", args)[0] == NULLPTR
+
+
+# ------------------------------------------------------------------------------------------------ finalize
+def _fin_args(aclnn, T_=12, K=2, H=7, E=3, mode=0, dtype=F32, **over):
+    ex = T(aclnn, over.get("ex_shape", (T_ * K, H) if mode in (0, 2) else (E, 4, H)), dtype)
+    idx = T(aclnn, over.get("idx_shape", (T_ * K,)), I32)
+    x1 = T(aclnn, over.get("x1_shape", (T_, H)), dtype) if over.get("x1", True) else None
+    x2 = T(aclnn, (T_, H), dtype) if over.get("x2", True) else None
+    bias = T(aclnn, over.get("bias_shape", (E, H)), dtype) if over.get("bias", True) else None
+    scales = T(aclnn, (T_, K), over.get("scale_dtype", dtype)) if over.get("scales", True) else None
+    eidx = T(aclnn, over.get("eidx_shape", (T_, K)), I32) if over.get("eidx", True) else None
+    out = T(aclnn, over.get("out_shape", (T_, H)), over.get("out_dtype", dtype))
+    return [ex.h, idx.h, x1.h if x1 else None, x2.h if x2 else None, bias.h if bias else None,
+            scales.h if scales else None, eidx.h if eidx else None, mode, out.h]
+
+
+def test_finalize_valid(aclnn):
+    for kw in [dict(), dict(mode=2), dict(mode=1), dict(mode=3), dict(dtype=BF16), dict(dtype=BF16, scale_dtype=F32),
+               dict(dtype=F16), dict(x1=False, x2=False, bias=False, eidx=False), dict(scales=False, K=1),
+               dict(T_=1024, K=4, H=30, E=10)]:
+        code, ws = _status(aclnn, "aclnnMoeFinalizeRoutingV2", _fin_args(aclnn, **kw))
+        assert code == 0 and ws == 0, (kw, ws)
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    (dict(mode=4), "drop_pad_mode should be [0,3]"),
+    (dict(mode=0, ex_shape=(3, 4, 7)), "2D tensor when drop_pad_mode is 0 or 2"),
+    (dict(mode=1, ex_shape=(24, 7)), "3D tensor when drop_pad_mode is 1 or 3"),
+    (dict(x1=False), "x2 parameter can't be inputted either"),
+    (dict(eidx=False), "expert_idx must exist when bias exist"),
+    (dict(x1_shape=(11, 7)), "dim 0 of x1"),
+    (dict(bias_shape=(3, 8)), "dim 1 of bias"),
+    (dict(bias_shape=(1, 7)), "E should be larger than or equal to K"),
+    (dict(eidx_shape=(12, 3)), "dim 1 of expert_idx"),
+    (dict(out_dtype=F16), "dtype of y should be same"),
+    (dict(out_shape=(12, 8)), "dim 1 of output"),
+    (dict(dtype=F16, scale_dtype=F32), "scales dtype"),
+])
+def test_finalize_invalid(aclnn, kw, fragment):
+    code, msg = _status(aclnn, "aclnnMoeFinalizeRoutingV2", _fin_args(aclnn, **kw))
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_second_phase_rejects_bad_workspace(aclnn):
+    """Phase 2 checks its arguments before touching the device."""
+    lib = aclnn.lib()
+    ws = ctypes.c_uint64(0)
+    ex = ctypes.c_void_p(None)
+    st = lib.aclnnMoeInitRoutingV2GetWorkspaceSize(*_routing_args(aclnn, flag=1), ctypes.byref(ws), ctypes.byref(ex))
+    assert st == 0 and ws.value > 0
+    st = lib.aclnnMoeInitRoutingV2(None, ws.value, ex, None)   # null workspace although bytes are required
+    assert st == NULLPTR
+    assert lib.aclnnMoeInitRoutingV2(None, 0, None, None) == NULLPTR  # null executor
