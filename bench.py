@@ -1,11 +1,16 @@
 """Benchmark of the quantized MoE expert-FFN path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline] [--calibration-copy]
 
 A step is one pass of the path (routing -> gate/up GEMM + SwiGLU + requant -> down GEMM -> finalize) over one batch of
 synthetic tokens whose inputs and expert weights are already resident in HBM.  Prints ONE JSON line: tokens/s for the
 whole pass, the roofline of the dominant kernel (the gate/up grouped GEMM) from HIP-event durations recorded inside the
 library during the timed steps, and the CPU oracle timed on a bounded sample of the same workload.
+
+--calibration-copy appends, after the timed region, a few launches of the library's plain 1 GiB copy kernel: under
+`rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` its counter readings give the factor that converts the counters to
+bytes.  roofline.traffic is read from the text summary of those counter runs under profiles/ (null when there is none
+for the workload): a counter run is a separate profiler pass and cannot happen inside this process.
 """
 import argparse
 import json
@@ -18,6 +23,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gmm_swiglu_{config}_hbm_traffic.txt")
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA (5.0 POP/s)
 
@@ -61,6 +67,17 @@ def _cpu_baseline(pkg, oracle, cfg, idx, wgt, xq, xs, ffn, sample_experts=4):
     return T / total, desc
 
 
+def _recorded_traffic(config_name):
+    """HBM bytes per launch of the gate/up GEMM from the committed counter summary ("traffic_bytes_per_launch: N")."""
+    path = TRAFFIC_FILE.format(config=config_name.split("_")[0])
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_launch:"):
+            return float(line.split(":", 1)[1])
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -68,6 +85,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (expert parallelism is a design note only); "
@@ -105,6 +123,13 @@ def main():
     elapsed = time.perf_counter() - t0
     kernels = aclnn.kernel_timer_report()
     aclnn.kernel_timer_enable(False)
+    if args.calibration_copy:
+        src = torch.empty(1 << 30, dtype=torch.int8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            aclnn.calibration_copy(dst, src)
+        torch.cuda.synchronize()
+        del src, dst
 
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = cfg.tokens / (elapsed / args.steps)
@@ -126,11 +151,11 @@ def main():
     t_mfma = gemm1_ops / (INT8_PEAK_TOPS * 1e12)
     if t_hbm >= t_mfma:
         roofline = {"bound": "hbm", "achieved": gemm1_bytes / (gemm1_ms * 1e-3) / 1e9 if gemm1_ms else None,
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac, "traffic": None}
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac, "traffic": _recorded_traffic(cfg.name)}
     else:
         roofline = {"bound": "mfma", "achieved": gemm1_ops / (gemm1_ms * 1e-3) / 1e12 if gemm1_ms else None,
-                    "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": None}
-    roofline.update({"kernel": "GroupedGemmKernel<kSwiglu> (gate/up GEMM + SwiGLU)", "kernel_ms": gemm1_ms,
+                    "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": _recorded_traffic(cfg.name)}
+    roofline.update({"kernel": "StreamGemmKernel<..., kSwiglu> (gate/up GEMM + SwiGLU; timer name gmm_swiglu)", "kernel_ms": gemm1_ms,
                      "algorithmic_bytes": gemm1_bytes, "algorithmic_ops": gemm1_ops,
                      "hbm_frac": hbm_frac, "mfma_frac": mfma_frac})
 

@@ -28,6 +28,14 @@ __attribute__((visibility("default"))) void opapiKernelTimerEnable(int enable);
  */
 __attribute__((visibility("default"))) int opapiKernelTimerReport(char* buf, size_t cap);
 
+/*
+ * Launches a plain copy kernel ("calibration_copy") moving `bytes` (a multiple of 16, both pointers 16-byte aligned)
+ * from src to dst on `stream`.  Its HBM traffic is known exactly (bytes read + bytes written), so reading a hardware
+ * traffic counter for it gives the factor that converts the counter's units to bytes for the other kernels.
+ * Returns 0, or an aclnn status code for bad arguments / a failed launch.
+ */
+__attribute__((visibility("default"))) int opapiCalibrationCopy(void* dst, const void* src, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -326,3 +326,14 @@ def kernel_timer_report():
         name, count, total = line.split()
         out[name] = (int(count), float(total))
     return out
+
+
+def calibration_copy(dst, src):
+    """Runs the library's plain copy kernel (include/opapi_profile.h) from src to dst, two same-sized device tensors."""
+    assert dst.is_contiguous() and src.is_contiguous() and dst.numel() * dst.element_size() == src.numel() * src.element_size()
+    l = lib()
+    l.opapiCalibrationCopy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    l.opapiCalibrationCopy.restype = ctypes.c_int
+    rc = l.opapiCalibrationCopy(dst.data_ptr(), src.data_ptr(), src.numel() * src.element_size(), _stream_ptr())
+    if rc != 0:
+        raise AclnnError("opapiCalibrationCopy", rc, last_error())

@@ -25,6 +25,7 @@ SOURCES = [
     "grouped_matmul_swiglu_quant.hip",
     "grouped_matmul_v4.hip",
     "moe_finalize_routing_v2.hip",
+    "calibration_copy.hip",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
