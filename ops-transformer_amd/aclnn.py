@@ -58,10 +58,13 @@ _PHASE1_SIGNATURES = {
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulV4GetWorkspaceSize":
         [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _VP, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulV5GetWorkspaceSize":
+        [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnMoeFinalizeRoutingV2GetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _U64P, _VPP],
 }
-_PHASE2 = ["aclnnMoeInitRoutingV2", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnMoeFinalizeRoutingV2"]
+_PHASE2 = ["aclnnMoeInitRoutingV2", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
+           "aclnnMoeFinalizeRoutingV2"]
 
 
 def lib():
@@ -89,6 +92,9 @@ def lib():
         l.aclCreateTensorList.restype = _VP
         l.aclDestroyTensorList.argtypes = [_VP]
         l.aclDestroyAclOpExecutor.argtypes = [_VP]
+        l.aclCreateIntArray.argtypes = [ctypes.POINTER(_I64), ctypes.c_uint64]
+        l.aclCreateIntArray.restype = _VP
+        l.aclDestroyIntArray.argtypes = [_VP]
         l.aclGetRecentErrMsg.restype = ctypes.c_char_p
         _lib = l
     return _lib
@@ -127,6 +133,7 @@ class _Handles:
     def __init__(self):
         self.tensors = []
         self.lists = []
+        self.int_arrays = []
 
     def tensor(self, t):
         if t is None:
@@ -144,8 +151,19 @@ class _Handles:
         self.lists.append(h)  # the list owns its tensors
         return h
 
+    def int_array(self, values):
+        if values is None:
+            return None
+        arr = (_I64 * max(len(values), 1))(*values)
+        h = lib().aclCreateIntArray(arr, len(values))
+        self.int_arrays.append(h)
+        return h
+
     def close(self):
         l = lib()
+        for h in self.int_arrays:
+            l.aclDestroyIntArray(h)
+        self.int_arrays = []
         for h in self.tensors:
             l.aclDestroyTensor(h)
         for h in self.lists:
@@ -262,9 +280,10 @@ def grouped_matmul_swiglu_quant(x, weight, group_list, weight_scale, x_scale, bi
 def grouped_matmul_v4(x, weight, bias=None, scale=None, offset=None, antiquant_scale=None, antiquant_offset=None,
                       per_token_scale=None, group_list=None, activation_input=None, activation_quant_scale=None,
                       activation_quant_offset=None, split_item=0, group_type=-1, group_list_type=0, act_type=0,
-                      output_dtype=None, out=None, workspace=None):
-    """aclnnGroupedMatmulV4.  x / weight / scale / per_token_scale / out are lists of tensors as in the reference.
-    Returns the list of outputs."""
+                      output_dtype=None, out=None, workspace=None, tuning_config=None):
+    """aclnnGroupedMatmulV4, or aclnnGroupedMatmulV5 when tuning_config (a list of ints whose first value is the expected
+    number of rows per expert) is given.  x / weight / scale / per_token_scale / out are lists of tensors as in the
+    reference.  Returns the list of outputs."""
     dev = x[0].device
     if out is None:
         if output_dtype is None:
@@ -277,11 +296,20 @@ def grouped_matmul_v4(x, weight, bias=None, scale=None, offset=None, antiquant_s
                 h.tensor_list(offset), h.tensor_list(antiquant_scale), h.tensor_list(antiquant_offset),
                 h.tensor_list(per_token_scale), h.tensor(group_list), h.tensor_list(activation_input),
                 h.tensor_list(activation_quant_scale), h.tensor_list(activation_quant_offset), split_item, group_type,
-                group_list_type, act_type, h.tensor_list(out), None, None]
-        _run_two_phase("aclnnGroupedMatmulV4", args, dev, workspace)
+                group_list_type, act_type]
+        if tuning_config is not None:
+            args.append(h.int_array(tuning_config))
+        args += [h.tensor_list(out), None, None]
+        _run_two_phase("aclnnGroupedMatmulV5" if tuning_config is not None else "aclnnGroupedMatmulV4", args, dev,
+                       workspace)
     finally:
         h.close()
     return out
+
+
+def grouped_matmul_v5(x, weight, tuning_config=(), **kwargs):
+    """aclnnGroupedMatmulV5: grouped_matmul_v4 plus the tuning hint (an empty list means "no hint")."""
+    return grouped_matmul_v4(x, weight, tuning_config=list(tuning_config), **kwargs)
 
 
 def moe_finalize_routing_v2(expanded_x, expanded_row_idx, x1=None, x2=None, bias=None, scales=None, expert_idx=None,

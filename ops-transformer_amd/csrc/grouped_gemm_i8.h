@@ -26,6 +26,7 @@ struct Problem {
     const void* groupList = nullptr; // device, int64 or int32, cumsum or counts
     bool groupListIsInt64 = true;
     GroupListKind groupListKind = GroupListKind::kCumsum;
+    int64_t expectedRowsPerGroup = 0; // > 0: caller's hint for the tile height; 0: use M / groups
     // epilogue
     Epilogue epilogue = Epilogue::kInt32;
     void* out = nullptr;             // kInt32 / kDequant: [M, N]

@@ -747,7 +747,9 @@ Plan MakePlan(const Problem& p) {
     const int64_t groups = p.groups > 0 ? p.groups : 1;
     // tile height: the mean group size plus a quarter, so that almost every group is covered by one m-tile and its
     // weights are streamed exactly once
-    const double want = static_cast<double>(p.M) / static_cast<double>(groups) * 1.25;
+    const double meanRows = p.expectedRowsPerGroup > 0 ? static_cast<double>(p.expectedRowsPerGroup)
+                                                       : static_cast<double>(p.M) / static_cast<double>(groups);
+    const double want = meanRows * 1.25;
     if (StreamOk(p)) {
         static const int kShapes[] = {32, 64, 96, 128, 160, 192, 256};
         plan.tileM = 256;

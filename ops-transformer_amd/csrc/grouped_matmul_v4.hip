@@ -10,7 +10,7 @@
 //   :1883-1916 groupListType 0/1 (2 = sparse list, not built), actType range
 // Widenings of this build: scale FLOAT with out BF16 is accepted; groupList may be INT32.
 // Group boundaries: grouped_matmul_utils.h:243-257.  The arithmetic is in grouped_gemm_i8.hip.
-#include "aclnnop/aclnn_grouped_matmul_v4.h"
+#include "aclnnop/aclnn_grouped_matmul_v5.h"
 
 #include <new>
 
@@ -54,15 +54,19 @@ constexpr int64_t kMaxGroupListTensor = 1024;
 
 }  // namespace
 
-extern "C" aclnnStatus aclnnGroupedMatmulV4GetWorkspaceSize(
+namespace {
+
+// Shared first phase of V4 and V5.  expectedRowsPerGroup > 0 is V5's tuning hint (tuningConfig[0]): the expected number
+// of rows per expert, which picks the tile height instead of the static mean M / groups.
+aclnnStatus PlanGroupedMatmul(
     const aclTensorList* x, const aclTensorList* weight, const aclTensorList* biasOptional,
     const aclTensorList* scaleOptional, const aclTensorList* offsetOptional, const aclTensorList* antiquantScaleOptional,
     const aclTensorList* antiquantOffsetOptional, const aclTensorList* perTokenScaleOptional,
     const aclTensor* groupListOptional, const aclTensorList* activationInputOptional,
     const aclTensorList* activationQuantScaleOptional, const aclTensorList* activationQuantOffsetOptional,
-    int64_t splitItem, int64_t groupType, int64_t groupListType, int64_t actType, aclTensorList* out,
-    aclTensorList* activationFeatureOutOptional, aclTensorList* dynQuantScaleOutOptional, uint64_t* workspaceSize,
-    aclOpExecutor** executor) {
+    int64_t splitItem, int64_t groupType, int64_t groupListType, int64_t actType, int64_t expectedRowsPerGroup,
+    aclTensorList* out, aclTensorList* activationFeatureOutOptional, aclTensorList* dynQuantScaleOutOptional,
+    uint64_t* workspaceSize, aclOpExecutor** executor) {
     using namespace opapi;
     ClearError();
     constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;
@@ -206,11 +210,58 @@ extern "C" aclnnStatus aclnnGroupedMatmulV4GetWorkspaceSize(
         p.scaleDtype = static_cast<int>(scale->dtype);
         p.rowScale = perToken != nullptr ? reinterpret_cast<const float*>(DataPtr(perToken)) : nullptr;
     }
+    p.expectedRowsPerGroup = expectedRowsPerGroup;
     ex->plan = gemm::MakePlan(p);
     ex->workspaceBytes = ex->plan.workspaceBytes;
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" aclnnStatus aclnnGroupedMatmulV4GetWorkspaceSize(
+    const aclTensorList* x, const aclTensorList* weight, const aclTensorList* biasOptional,
+    const aclTensorList* scaleOptional, const aclTensorList* offsetOptional, const aclTensorList* antiquantScaleOptional,
+    const aclTensorList* antiquantOffsetOptional, const aclTensorList* perTokenScaleOptional,
+    const aclTensor* groupListOptional, const aclTensorList* activationInputOptional,
+    const aclTensorList* activationQuantScaleOptional, const aclTensorList* activationQuantOffsetOptional,
+    int64_t splitItem, int64_t groupType, int64_t groupListType, int64_t actType, aclTensorList* out,
+    aclTensorList* activationFeatureOutOptional, aclTensorList* dynQuantScaleOutOptional, uint64_t* workspaceSize,
+    aclOpExecutor** executor) {
+    return PlanGroupedMatmul(x, weight, biasOptional, scaleOptional, offsetOptional, antiquantScaleOptional,
+                             antiquantOffsetOptional, perTokenScaleOptional, groupListOptional, activationInputOptional,
+                             activationQuantScaleOptional, activationQuantOffsetOptional, splitItem, groupType,
+                             groupListType, actType, /*expectedRowsPerGroup=*/0, out, activationFeatureOutOptional,
+                             dynQuantScaleOutOptional, workspaceSize, executor);
+}
+
+// V5 = V4 plus tuningConfigOptional, whose first value is the expected number of tokens per expert
+// (reference: aclnn_grouped_matmul.cpp:1957-1992; it only steers tiling, never results).
+extern "C" aclnnStatus aclnnGroupedMatmulV5GetWorkspaceSize(
+    const aclTensorList* x, const aclTensorList* weight, const aclTensorList* biasOptional,
+    const aclTensorList* scaleOptional, const aclTensorList* offsetOptional, const aclTensorList* antiquantScaleOptional,
+    const aclTensorList* antiquantOffsetOptional, const aclTensorList* perTokenScaleOptional,
+    const aclTensor* groupListOptional, const aclTensorList* activationInputOptional,
+    const aclTensorList* activationQuantScaleOptional, const aclTensorList* activationQuantOffsetOptional,
+    int64_t splitItem, int64_t groupType, int64_t groupListType, int64_t actType, aclIntArray* tuningConfigOptional,
+    aclTensorList* out, aclTensorList* activationFeatureOutOptional, aclTensorList* dynQuantScaleOutOptional,
+    uint64_t* workspaceSize, aclOpExecutor** executor) {
+    int64_t expected = 0;
+    if (tuningConfigOptional != nullptr && !tuningConfigOptional->values.empty() &&
+        tuningConfigOptional->values[0] > 0) {
+        expected = tuningConfigOptional->values[0];
+    }
+    return PlanGroupedMatmul(x, weight, biasOptional, scaleOptional, offsetOptional, antiquantScaleOptional,
+                             antiquantOffsetOptional, perTokenScaleOptional, groupListOptional, activationInputOptional,
+                             activationQuantScaleOptional, activationQuantOffsetOptional, splitItem, groupType,
+                             groupListType, actType, expected, out, activationFeatureOutOptional,
+                             dynQuantScaleOutOptional, workspaceSize, executor);
+}
+
+extern "C" aclnnStatus aclnnGroupedMatmulV5(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
+                                            aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
 }
 
 extern "C" aclnnStatus aclnnGroupedMatmulV4(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,

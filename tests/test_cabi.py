@@ -32,6 +32,7 @@ def test_headers_declare_the_expected_entry_points():
     for required in ["aclnnMoeInitRoutingV2GetWorkspaceSize", "aclnnMoeInitRoutingV2",
                      "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize", "aclnnGroupedMatmulSwigluQuant",
                      "aclnnGroupedMatmulV4GetWorkspaceSize", "aclnnGroupedMatmulV4",
+                     "aclnnGroupedMatmulV5GetWorkspaceSize", "aclnnGroupedMatmulV5",
                      "aclnnMoeFinalizeRoutingV2GetWorkspaceSize", "aclnnMoeFinalizeRoutingV2",
                      "aclCreateTensor", "aclDestroyTensor", "aclCreateTensorList", "aclDestroyTensorList", "aclrtMalloc",
                      "aclrtMemcpy", "aclGetRecentErrMsg", "ResetCacheThreadLocal", "opapiKernelTimerEnable",
@@ -231,6 +232,38 @@ def test_gmm_reserved_arguments_and_nulls(aclnn):
     args = _gmm_args(aclnn)
     args[16] = None
     assert _status(aclnn, "aclnnGroupedMatmulV4", args)[0] == NULLPTR
+
+
+def test_gmm_v5_takes_a_tuning_hint(aclnn):
+    """V5 = V4 + tuningConfigOptional (absent, empty or a positive expected-rows hint); same validation as V4."""
+    lib = aclnn.lib()
+    for values in (None, [], [64], [4096, 1]):
+        args = _gmm_args(aclnn)
+        arr = None
+        if values is not None:
+            buf = (ctypes.c_int64 * max(len(values), 1))(*values)
+            arr = lib.aclCreateIntArray(buf, len(values))
+        args = args[:16] + [arr] + args[16:]
+        code, ws = _status(aclnn, "aclnnGroupedMatmulV5", args)
+        assert code == 0 and ws > 0, (values, ws)
+    args = _gmm_args(aclnn, group_type=2)
+    args = args[:16] + [None] + args[16:]
+    code, msg = _status(aclnn, "aclnnGroupedMatmulV5", args)
+    assert code == INVALID and "groupType 0" in msg
+
+
+def test_reference_examples_compile_and_link_unmodified():
+    """The four example programs of the reference for the operators on the path build against include/ and link to
+    libcust_opapi.so without a change (needs the reference checkout; the binaries are run by the GPU tests)."""
+    import subprocess
+    if not os.path.isdir("/root/reference/moe/moe_init_routing_v2/examples"):
+        pytest.skip("reference sources are not present on this machine")
+    res = subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "-B", "ref_examples"], stdout=subprocess.PIPE,
+                         stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout
+    for name in ("test_aclnn_moe_init_routing_v2", "test_aclnn_grouped_matmul_swiglu_quant", "test_aclnn_grouped_matmul",
+                 "test_aclnn_moe_finalize_routing_v2"):
+        assert os.access(os.path.join(ROOT, "oracle", "_ref", "examples", name), os.X_OK), name
 
 
 # ------------------------------------------------------------------------------------------------ finalize

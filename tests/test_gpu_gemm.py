@@ -159,3 +159,17 @@ def test_swiglu_empty_group_list_is_noop(aclnn, dev):
     y, ys = aclnn.grouped_matmul_swiglu_quant(x, w, gl, torch.ones((2, 64), device=dev), torch.ones((4,), device=dev))
     torch.cuda.synchronize()
     assert y.shape == (4, 32)
+
+
+@pytest.mark.parametrize("hint", [[], [16], [96], [4096]])
+def test_v5_tuning_hint_changes_tiling_not_results(aclnn, oracle, dev, hint):
+    """aclnnGroupedMatmulV5's tuningConfig picks another tile height; the int32 accumulators stay bit-exact."""
+    rng = np.random.default_rng(55)
+    M, K, N, E = 900, 512, 320, 6
+    x, wt, cumsum = _problem(rng, M, K, N, E, "ragged")
+    ref = oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)
+    out = aclnn.grouped_matmul_v5([torch.from_numpy(x).to(dev)], [_weight_views(wt, dev, "kmajor")], tuning_config=hint,
+                                  group_list=torch.from_numpy(cumsum).to(dev), split_item=3, group_type=0,
+                                  group_list_type=0, act_type=0, output_dtype=torch.int32)[0]
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), ref)
