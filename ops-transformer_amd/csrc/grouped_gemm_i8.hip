@@ -216,6 +216,13 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                                              int waveRow0, int waveN, int l32, int lhi, int tid,
                                              const float* ldsRowScale, float* ldsRowMax) {
     const int32_t rows = t.rows, rowBase = t.rowBase, group = t.group;
+    // The row / address arithmetic below depends only on the lane; hoisted out of the persistent tile loop it would
+    // stay alive across the whole kernel and spill, and a reload in here waits for every store issued so far.  An
+    // opaque per-call zero folded into the lane index keeps the arithmetic inside the epilogue.
+    int opaqueZero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(opaqueZero));
+    lhi += opaqueZero;
+    l32 += opaqueZero;
     if (kEpi == Epilogue::kInt32 || kEpi == Epilogue::kDequant) {
         const bool hasRowScale = a.rowScale != nullptr;
         const int32_t n0 = t.colBase + 64 * waveN + l32;  // column block 0; block 1 is 32 columns further
