@@ -328,6 +328,17 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
     }
 }
 
+// Calls f(std::integral_constant<int, n>) for n = count clamped into 0..kMax.
+template <int kMax, typename F>
+__device__ __forceinline__ void ForCount(int count, F& f) {
+    if constexpr (kMax == 0) {
+        f(std::integral_constant<int, 0>{});
+    } else {
+        if (count >= kMax) f(std::integral_constant<int, kMax>{});
+        else ForCount<kMax - 1>(count, f);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------- fast path: LDS-DMA ring
 // kStep = k-bytes per ring stage: 128 streams weights in whole 128-byte lines (best HBM efficiency) when three such
 // stages fit in LDS, 64 allows a deeper ring for the tall tiles.
@@ -443,15 +454,15 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     const int kSteps = a.K / kStep;
 
     // ---- issue side: runs kStages - 1 steps ahead of the compute side, across tile boundaries ----
+    const uint32_t ldsBase = LdsAddress(lds);
     TileInfo iss = cur;
     int64_t issLocal = local;
     int issStep = 0;
     const char* issX = nullptr;
     const char* issW = nullptr;
     uint32_t laneOff[Cfg::kMaxPerWave];
-    int dmaPerStage = 0;  // DMA instructions this wave issues per stage
-#pragma unroll
-    for (int q = 0; q < Cfg::kMaxPerWave; ++q) dmaPerStage += (wave + q * Cfg::kWaves < Cfg::kInstr) ? 1 : 0;
+    // Every wave issues exactly kMaxPerWave DMA instructions per stage: slots past the last instruction repeat it (same
+    // bytes to the same place), which keeps the issue code free of branches and the vmcnt arithmetic uniform.
 
     auto setupIssue = [&]() {
         issX = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(iss.rowBase) * a.K;
@@ -461,7 +472,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         const int slot = lane % Cfg::kChunksPerRow;
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
-            const int j = wave + q * Cfg::kWaves;
+            const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
             if (j < Cfg::kInstrA) {
                 // rows past the tile's last row are never used: such lanes re-read the last real row (same cache
                 // lines as its own lanes), and an instruction wholly past it reads one chunk, so the number of DMAs
@@ -478,12 +489,12 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         }
     };
     auto issueStage = [&](int ring) {
-        char* const dst = lds + ring * kStageBytes;
+        const uint32_t dst = ldsBase + ring * kStageBytes;
         const int kOff = issStep * kStep;
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
-            const int j = wave + q * Cfg::kWaves;
-            if (j < Cfg::kInstr) DmaToLds16((j < Cfg::kInstrA ? issX : issW) + kOff, laneOff[q], dst + j * 1024);
+            const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
+            DmaToLdsAddr16((j < Cfg::kInstrA ? issX : issW) + kOff, laneOff[q], dst + j * 1024);
         }
         if (++issStep == kSteps) {
             // move to this workgroup's next tile; past the last one the same tile is fetched again into ring slots
@@ -507,8 +518,12 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         ldsRowScale[tid] = a.rowScale[cur.rowBase + (tid < cur.rows ? tid : cur.rows - 1)];
     }
 
-    const int waveRow0 = waveM * 32 * kSub0;
-    const int mySub = waveM == 0 ? kSub0 : kSub1;  // MFMA tiles of this wave
+    // The tile's real rows (rounded up to whole 32-row MFMA tiles) are split between the two wave rows tile by tile:
+    // wave row 0 takes the first half (rounded up), wave row 1 the rest, and MFMA tiles that hold no real row are never
+    // computed -- on the memory-bound shapes the matrix pipe's power is what is worth saving.  The k loop is
+    // instantiated once per MFMA-tile count (0..kSub0) so that its body stays straight-line code.
+    int waveRow0 = 0;  // first tile row of this wave
+    int mySub = 0;     // MFMA tiles of this wave in the current tile
     const int bRow0 = kSwiglu ? 32 * waveN : 64 * waveN;
     const int bRowStep = kSwiglu ? kTileN / 2 : 32;
     v16i acc[kSubM][2];
@@ -527,33 +542,56 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
 
-#pragma unroll 1
-        for (int step = 0; step < kSteps; ++step) {
-            // the oldest stage in flight has landed once at most (kStages - 2) stages' worth of this wave's DMAs remain
-            if (dmaPerStage == Cfg::kMaxPerWave) WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
-            else WaitVmcnt<(kStages - 2) * (Cfg::kMaxPerWave - 1)>();
-            __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
+        // One k-step of a wave with kMy MFMA tiles: straight-line code, the operands of k-slice ks + 1 are read
+        // from LDS before the MFMAs of k-slice ks are issued, and the refill of the stage freed by the barrier goes out
+        // behind the first block of MFMAs (its scalar address work then runs in the shadow of the matrix pipe).
+        auto computeStep = [&](auto myTag) {
+            constexpr int kMy = decltype(myTag)::value;
             const char* const A = lds + ring * kStageBytes;
             const char* const B = A + kTileM * kStep;
-#pragma unroll
-            for (int ks = 0; ks < kStep / 32; ++ks) {
+            constexpr int kSlices = kStep / 32;
+            v4i bf[2][2];
+            v4i af[2][kMy > 0 ? kMy : 1];
+            auto loadSlice = [&](int ks, int buf) {
+                if (kMy == 0) return;
                 const int chunk = 2 * ks + lhi;
-                const v4i b0 = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + l32, chunk));
-                const v4i b1 = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + bRowStep + l32, chunk));
+                bf[buf][0] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + l32, chunk));
+                bf[buf][1] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + bRowStep + l32, chunk));
 #pragma unroll
-                for (int mi = 0; mi < kSubM; ++mi) {
-                    if (mi < kSub1 || waveM == 0) {  // compile-time true for the tiles both wave rows have
-                        const v4i av = *reinterpret_cast<const v4i*>(A + LdsOffset<kStep>(waveRow0 + mi * 32 + l32, chunk));
-                        acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b0, acc[mi][0], 0, 0, 0);
-                        acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, acc[mi][1], 0, 0, 0);
-                    }
+                for (int mi = 0; mi < kMy; ++mi) {
+                    af[buf][mi] = *reinterpret_cast<const v4i*>(A + LdsOffset<kStep>(waveRow0 + mi * 32 + l32, chunk));
                 }
-                // The refill of the stage freed by the barrier is issued behind the first block of MFMAs: its scalar
-                // address work then runs in the shadow of the matrix pipe instead of in front of it.
+            };
+            loadSlice(0, 0);
+#pragma unroll
+            for (int ks = 0; ks < kSlices; ++ks) {
+                if (ks + 1 < kSlices) loadSlice(ks + 1, (ks + 1) & 1);
+#pragma unroll
+                for (int mi = 0; mi < kMy; ++mi) {
+                    acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][0], acc[mi][0], 0, 0, 0);
+                    acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][1], acc[mi][1], 0, 0, 0);
+                }
                 if (ks == 0) issueStage(ring == 0 ? kStages - 1 : ring - 1);
             }
-            ring = ring + 1 == kStages ? 0 : ring + 1;
+        };
+
+        auto runTile = [&](auto myTag) {
+#pragma unroll 1
+            for (int step = 0; step < kSteps; ++step) {
+                // the oldest stage in flight has landed once at most (kStages - 2) stages' worth of this wave's DMAs remain
+                WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
+                __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
+                computeStep(myTag);
+                ring = ring + 1 == kStages ? 0 : ring + 1;
+            }
+        };
+        {
+            const int active = (cur.rows + 31) >> 5;                       // MFMA tiles with real rows, 1..kSub0+kSub1
+            const int share0 = Cfg::kWavesM == 2 ? (active + 1) >> 1 : active;  // wave row 0's share
+            waveRow0 = waveM == 0 ? 0 : 32 * share0;
+            mySub = waveM == 0 ? share0 : active - share0;
         }
+        ForCount<kSub0>(mySub, runTile);
 
         TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
         // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
