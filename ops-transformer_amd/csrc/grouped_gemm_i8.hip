@@ -238,6 +238,37 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
         const bool pairStores = kEpi == Epilogue::kDequant && a.outDtype != 0 && (a.N & 1) == 0 &&
                                 t.colBase + 64 * waveN + 64 <= a.N;  // wave-uniform
         const bool oddLane = (l32 & 1) != 0;
+        if (kEpi == Epilogue::kDequant && a.outDtype == 27 && pairStores) {
+            // The common case (bf16 output, whole column pairs) without per-element dtype dispatch: row scales come
+            // from LDS four at a time, every lane stores one 32-bit word per accumulator pair through a
+            // (uniform row pointer + 32-bit lane offset) address.
+            uint16_t* const outTile = static_cast<uint16_t*>(a.out) + static_cast<int64_t>(rowBase + waveRow0) * a.N;
+            const int32_t laneOff = 4 * lhi * a.N + (oddLane ? n0 + 31 : n0);
+#pragma unroll
+            for (int mi = 0; mi < kSubM; ++mi) {
+                const int rTop = waveRow0 + 32 * mi;
+                if (mi >= mySub || rTop >= rows) continue;
+                const bool full = rTop + 32 <= rows;  // wave-uniform: no row checks for whole MFMA tiles
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float4 rs = make_float4(1.0f, 1.0f, 1.0f, 1.0f);  // multiplying by 1 is exact
+                    if (hasRowScale) rs = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
+                    const float rsv[4] = {rs.x, rs.y, rs.z, rs.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int v = 4 * q + i;
+                        const Float2 f = {__fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), sc0), rsv[i]),
+                                          __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), sc1), rsv[i])};
+                        const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));
+                        const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
+                        const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
+                        uint16_t* const rowPtr = outTile + static_cast<int64_t>(32 * mi + 8 * q + i) * a.N;
+                        if (full || rTop + 8 * q + 4 * lhi + i < rows) *reinterpret_cast<uint32_t*>(rowPtr + laneOff) = word;
+                    }
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int mi = 0; mi < kSubM; ++mi) {
             if (mi >= mySub || waveRow0 + 32 * mi >= rows) continue;
@@ -293,9 +324,64 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
             scA = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + j, a.scaleDtype);
             scB = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + a.halfN + j, a.scaleDtype);
         }
+        const bool wholeColumns = t.colBase + 32 * waveN + 32 <= a.halfN;  // wave-uniform
 #pragma unroll
         for (int mi = 0; mi < kSubM; ++mi) {
             if (mi >= mySub) continue;  // wave-uniform
+            const int rTop = waveRow0 + 32 * mi;
+            if (wholeColumns && rTop < rows) {
+                // Fast form for whole column blocks: row scales four at a time, no column checks, and the 16 row
+                // maxima of the MFMA tile reduced across the 32 lanes by a halving butterfly (16 exchanges, not 80).
+                const bool full = rTop + 32 <= rows;  // wave-uniform
+                float* const sTile = a.sOut + static_cast<int64_t>(rowBase + rTop) * a.halfN;
+                const int32_t laneOff = 4 * lhi * a.halfN + j;
+                float m[16];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 xs4 = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
+                    const float xsv[4] = {xs4.x, xs4.y, xs4.z, xs4.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int v = 4 * q + i;
+                        const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), xsv[i]), scA);
+                        const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xsv[i]), scB);
+                        float sv = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
+                        const bool ok = full || rTop + 8 * q + 4 * lhi + i < rows;
+                        if (ok) sTile[static_cast<int64_t>(8 * q + i) * a.halfN + laneOff] = sv;
+                        m[v] = ok ? fabsf(sv) : 0.0f;
+                    }
+                }
+                // lanes l and l ^ 16: one instruction trades the upper-row half of m[i] for the lower-row half of
+                // m[i + 8]; afterwards lanes 0..15 of each half-wave own v = i and lanes 16..31 own v = i + 8
+                typedef unsigned int Uint2 __attribute__((ext_vector_type(2)));
+                float k8[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const Uint2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(m[i]), __float_as_uint(m[i + 8]), false, false);
+                    k8[i] = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                }
+                const bool b3 = (l32 & 8) != 0, b2 = (l32 & 4) != 0, b1 = (l32 & 2) != 0;
+                float k4[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {  // partner l ^ 8: lanes with bit 3 clear keep i, the others i + 4
+                    const float send = b3 ? k8[i] : k8[i + 4];
+                    k4[i] = fmaxf(b3 ? k8[i + 4] : k8[i], __shfl_xor(send, 8, 64));
+                }
+                float k2[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const float send = b2 ? k4[i] : k4[i + 2];
+                    k2[i] = fmaxf(b2 ? k4[i + 2] : k4[i], __shfl_xor(send, 4, 64));
+                }
+                const float send1 = b1 ? k2[0] : k2[1];
+                float k1 = fmaxf(b1 ? k2[1] : k2[0], __shfl_xor(send1, 2, 64));
+                k1 = fmaxf(k1, __shfl_xor(k1, 1, 64));
+                // the lane pair (2p, 2p + 1) of a half-wave now holds the maximum of accumulator index v = p:
+                // bit 4 of the lane chose bit 3 of v, bit 3 -> bit 2, bit 2 -> bit 1, bit 1 -> bit 0
+                const int v = l32 >> 1;
+                if ((l32 & 1) == 0) ldsRowMax[waveN * kTileM + rTop + 8 * (v / 4) + 4 * lhi + (v % 4)] = k1;
+                continue;
+            }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int r = waveRow0 + 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
@@ -1017,7 +1103,7 @@ __global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a, const int
     constexpr bool kSwiglu = kEpi == Epilogue::kSwiglu;
     __shared__ __attribute__((aligned(16))) char ldsA[kTileM * kGenStep];
     __shared__ __attribute__((aligned(16))) char ldsB[kTileN * kGenStep];
-    __shared__ float ldsRowScale[kTileM];
+    __shared__ __attribute__((aligned(16))) float ldsRowScale[kTileM];
     __shared__ float ldsRowMax[kWavesN * kTileM];
 
     const int tid = threadIdx.x;
