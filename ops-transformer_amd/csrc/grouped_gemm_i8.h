@@ -46,6 +46,7 @@ struct Plan {
     int wavesM = 1;         // 1 or 2 wave rows
     int subTilesM = 1;      // 32-row MFMA tiles per wave
     int64_t maxTiles = 0;   // launch bound on workgroups
+    int32_t maxMTiles = 0;  // upper bound on m-tiles over all groups (M / tileM + groups)
     int32_t tilesN = 0;
     uint64_t offSched = 0, offRowMax = 0, offS = 0;
     uint64_t workspaceBytes = 0;

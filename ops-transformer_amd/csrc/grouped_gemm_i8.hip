@@ -51,8 +51,10 @@ constexpr int kMaxGroups = 1024;
 constexpr int kLdsBudget = 160 * 1024;
 
 // ---------------------------------------------------------------------------------------------- scheduling table
-// int32 layout: [0] total rows covered by groups, [1] total m-tiles, [2..2+G) row start, [..+G) rows, [..+G+1) m-tile prefix
-__host__ __device__ inline int SchedInts(int groups) { return 2 + 3 * groups + 1; }
+// int32 layout: [0] total rows covered by groups, [1] total m-tiles, [2..2+G) row start, [..+G) rows, [..+G+1) m-tile prefix,
+// then one entry per m-tile (at most maxMTiles of them): the group it belongs to, so that the GEMM kernels find a
+// tile's group with one load instead of a binary search of dependent loads
+__host__ __device__ inline int SchedInts(int groups, int maxMTiles) { return 2 + 3 * groups + 1 + maxMTiles; }
 
 struct SchedArgs {
     const void* groupList;
@@ -61,6 +63,7 @@ struct SchedArgs {
     int32_t groupListIsInt64;
     int32_t isCount;
     int32_t tileM;
+    int32_t maxMTiles;
     int64_t M;
 };
 
@@ -119,6 +122,20 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
             a.sched[1] = tileInc;
         }
     }
+    // group of every m-tile: scan[] still holds the inclusive m-tile prefix (zero-tile groups repeat their
+    // predecessor's value); m-tile m belongs to the first group whose inclusive prefix exceeds m
+    scan[t] = t < a.groups ? tileInc : 0x7fffffff;
+    __syncthreads();
+    const int32_t totalMTiles = scan[a.groups - 1];
+    int32_t* const groupOfMTile = tilePrefix + a.groups + 1;
+    for (int32_t m = t; m < totalMTiles && m < a.maxMTiles; m += 1024) {
+        int lo = -1, hi = a.groups - 1;  // scan[hi] > m always holds, scan[lo] <= m (lo = -1: nothing before)
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (scan[mid] > m) hi = mid; else lo = mid;
+        }
+        groupOfMTile[m] = hi;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------- shared device code
@@ -164,11 +181,7 @@ __device__ __forceinline__ TileInfo DecodeTile(const KernelArgs& a, const int32_
     const int32_t* const rowCountTbl = rowStartTbl + a.groups;
     const int32_t* const tilePrefix = rowCountTbl + a.groups;
     const int32_t q = static_cast<int32_t>(logical / a.tilesN);
-    int lo = 0, hi = a.groups;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (tilePrefix[mid] <= q) lo = mid; else hi = mid;
-    }
+    const int lo = tilePrefix[a.groups + 1 + q];  // group of m-tile q
     const int32_t inGroup = static_cast<int32_t>(logical - static_cast<int64_t>(tilePrefix[lo]) * a.tilesN);
     const int32_t tilesM = tilePrefix[lo + 1] - tilePrefix[lo];
     const int32_t band = inGroup / (kGroupM * a.tilesN);
@@ -1367,11 +1380,12 @@ Plan MakePlan(const Problem& p) {
     const int64_t colsPerTile = p.epilogue == Epilogue::kSwiglu ? kTileN / 2 : kTileN;
     plan.tilesN = static_cast<int32_t>((cols + colsPerTile - 1) / colsPerTile);
     const int64_t maxMTiles = p.M / plan.tileM + groups;
+    plan.maxMTiles = static_cast<int32_t>(maxMTiles);
     // round up so that every XCD's share [xcd * ceil(total/8), ...) is covered by the launch
     plan.maxTiles = (maxMTiles * plan.tilesN + kXcds - 1) / kXcds * kXcds;
     uint64_t off = 0;
     plan.offSched = off;
-    off += Align256(static_cast<uint64_t>(SchedInts(static_cast<int>(groups))) * 4);
+    off += Align256(static_cast<uint64_t>(SchedInts(static_cast<int>(groups), plan.maxMTiles)) * 4);
     if (p.epilogue == Epilogue::kSwiglu) {
         plan.offRowMax = off;
         off += Align256(static_cast<uint64_t>(p.M) * 4 * static_cast<uint64_t>(plan.tilesN));
@@ -1398,6 +1412,7 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     sa.groupListIsInt64 = p.groupListIsInt64 ? 1 : 0;
     sa.isCount = p.groupListKind == GroupListKind::kCount ? 1 : 0;
     sa.tileM = plan.tileM;
+    sa.maxMTiles = plan.maxMTiles;
     sa.M = p.M;
     {
         opapi::KernelTimer timer("gmm_schedule", stream);
