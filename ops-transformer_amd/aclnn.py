@@ -54,6 +54,8 @@ _VPP = ctypes.POINTER(ctypes.c_void_p)
 _PHASE1_SIGNATURES = {
     "aclnnMoeInitRoutingV2GetWorkspaceSize":
         [_VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnMoeInitRoutingV3GetWorkspaceSize":
+        [_VP, _VP, _VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _I64, _VP, _I64, _VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulV4GetWorkspaceSize":
@@ -63,7 +65,7 @@ _PHASE1_SIGNATURES = {
     "aclnnMoeFinalizeRoutingV2GetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _U64P, _VPP],
 }
-_PHASE2 = ["aclnnMoeInitRoutingV2", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
+_PHASE2 = ["aclnnMoeInitRoutingV2", "aclnnMoeInitRoutingV3", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
            "aclnnMoeFinalizeRoutingV2"]
 
 
@@ -253,6 +255,32 @@ def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_n
     finally:
         h.close()
     return expanded_x, expanded_row_idx, count_out, before_out
+
+
+def moe_init_routing_v3(x, expert_idx, scale=None, expert_num=0, expert_tokens_num_type=1, quant_mode=-1,
+                        active_expert_range=None, row_idx_type=1, active_num=-1, out=None, workspace=None):
+    """aclnnMoeInitRoutingV3 (dropless).  Returns (expandedX, expandedRowIdx, tokenCounts int64, expandedScale or None)."""
+    T, H = x.shape
+    K = expert_idx.shape[1]
+    dev = x.device
+    start, end = (0, expert_num) if active_expert_range is None else active_expert_range
+    if out is not None:
+        expanded_x, row_idx, counts, expanded_scale = out
+    else:
+        expanded_x = torch.zeros((T * K, H), dtype=x.dtype, device=dev)
+        row_idx = torch.empty((T * K,), dtype=torch.int32, device=dev)
+        counts = torch.zeros((expert_num, 2) if expert_tokens_num_type == 2 else (end - start,), dtype=torch.int64, device=dev)
+        expanded_scale = None if scale is None else torch.zeros((T * K,), dtype=torch.float32, device=dev)
+    h = _Handles()
+    try:
+        args = [h.tensor(x), h.tensor(expert_idx), h.tensor(scale), None, active_num, 0, expert_num, 0,
+                expert_tokens_num_type, True, quant_mode,
+                None if active_expert_range is None else h.int_array(list(active_expert_range)), row_idx_type,
+                h.tensor(expanded_x), h.tensor(row_idx), h.tensor(counts), h.tensor(expanded_scale)]
+        _run_two_phase("aclnnMoeInitRoutingV3", args, dev, workspace)
+    finally:
+        h.close()
+    return expanded_x, row_idx, counts, expanded_scale
 
 
 def grouped_matmul_swiglu_quant(x, weight, group_list, weight_scale, x_scale, bias=None, offset=None, out=None,

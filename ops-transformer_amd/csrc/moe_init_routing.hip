@@ -1,4 +1,5 @@
-// aclnnMoeInitRoutingV2 for gfx950: top-k expansion, stable sort by expert, inverse map, per-expert counts, row gather.
+// aclnnMoeInitRoutingV2 and aclnnMoeInitRoutingV3 for gfx950: top-k expansion, stable sort by expert, inverse map,
+// per-expert counts, row gather (V3: expert range filter, int64 counts, gather- or scatter-type index, scale gather).
 //
 // Reference behaviour restated (not its structure): moe/moe_init_routing_v2/op_kernel/
 //   moe_v2_sort_one_core.h:64-113, moe_v2_sort_multi_core.h:498-504   stable ascending key/value sort of expert ids
@@ -22,6 +23,7 @@
 #include "opapi_common.h"
 
 #include "aclnnop/aclnn_moe_init_routing_v2.h"
+#include "aclnnop/aclnn_moe_init_routing_v3.h"
 
 namespace {
 
@@ -169,9 +171,11 @@ __global__ __launch_bounds__(1024) void DigitScanKernel(SortPass p, CountOutputs
 }
 
 struct InverseMap {
-    int32_t* expandedRowIdx;  // nullptr unless this is the last pass
+    int32_t* expandedRowIdx;  // scatter-type map [source] -> destination; nullptr unless this is the last pass
     int32_t dropPad;          // 1: destination is e*capacity + rank or -1
     int32_t capacity;
+    int32_t* gatherIdx;       // gather-type map [destination] -> source, or nullptr
+    int32_t dropFrom;         // destinations at or beyond binBase[dropFrom] are dropped (-1 in both maps); < 0: none
 };
 
 __global__ __launch_bounds__(kSortThreads) void DigitScatterKernel(SortPass p, InverseMap im) {
@@ -200,14 +204,16 @@ __global__ __launch_bounds__(kSortThreads) void DigitScatterKernel(SortPass p, I
             const int32_t payload = p.payloadIn != nullptr ? p.payloadIn[i] : static_cast<int32_t>(i);
             if (p.keysOut != nullptr) p.keysOut[dst] = key;
             if (p.payloadOut != nullptr) p.payloadOut[dst] = payload;
+            const bool dropped = im.dropFrom >= 0 && dst >= p.binBase[im.dropFrom];
             if (im.expandedRowIdx != nullptr) {
                 int32_t row = dst;
                 if (im.dropPad) {
                     const int32_t rank = dst - p.binBase[digit];
                     row = rank < im.capacity ? static_cast<int32_t>(digit) * im.capacity + rank : -1;
                 }
-                im.expandedRowIdx[payload] = row;
+                im.expandedRowIdx[payload] = dropped ? -1 : row;
             }
+            if (im.gatherIdx != nullptr) im.gatherIdx[dst] = dropped ? -1 : payload;
         }
     }
 }
@@ -239,6 +245,8 @@ struct GatherArgs {
     int64_t tokens;
     int32_t topK;
     int64_t activeRows;  // destinations at or beyond this row are not written
+    const float* scale;    // optional per-token scale, routed with the rows: expandedScale[destination] = scale[token]
+    float* expandedScale;
 };
 
 constexpr int kGatherThreads = 256;
@@ -252,6 +260,13 @@ __global__ __launch_bounds__(kGatherThreads) void GatherRowsKernel(GatherArgs a)
     const int kCached = a.topK < kMaxCachedK ? a.topK : kMaxCachedK;
     if (threadIdx.x < kCached) dsts[threadIdx.x] = a.expandedRowIdx[n * a.topK + threadIdx.x];
     __syncthreads();
+    if (a.scale != nullptr) {
+        const float s = a.scale[n];
+        for (int j = threadIdx.x; j < a.topK; j += kGatherThreads) {
+            const int64_t d = j < kMaxCachedK ? dsts[j] : a.expandedRowIdx[n * a.topK + j];
+            if (d >= 0 && d < a.activeRows) a.expandedScale[d] = s;
+        }
+    }
     const int64_t vecs = a.rowBytes / static_cast<int64_t>(sizeof(Vec));
     const Vec* src = reinterpret_cast<const Vec*>(a.x + n * a.rowBytes);
     for (int64_t v = threadIdx.x; v < vecs; v += kGatherThreads) {
@@ -278,6 +293,79 @@ __global__ __launch_bounds__(kGatherThreads) void ZeroUnusedCapacityKernel(char*
     for (int64_t v = threadIdx.x; v < vecs; v += kGatherThreads) dst[v] = zero;
 }
 
+// V3: ids inside [start, end) become 0 .. end-start-1, everything else the sentinel end-start, which sorts last.
+__global__ void RemapKeysKernel(const int32_t* ids, int32_t* keys, int64_t total, int32_t start, int32_t end) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int32_t id = ids[i];
+    keys[i] = (id >= start && id < end) ? id - start : end - start;
+}
+
+// V3 token-count output (int64) from the int32 per-expert counts of the active range.
+// mode 0: cumsum, 1: count, 2: key/value pairs (expert id, count) of the non-empty experts, zero-filled behind them.
+struct CountV3Args {
+    const int32_t* counts;  // [active]; nullptr: every count is zero
+    int64_t* out;
+    int32_t active;
+    int32_t expertStart;
+    int32_t mode;
+    int32_t kvPairs;        // pairs the key/value buffer holds
+};
+
+__global__ __launch_bounds__(1024) void CountV3Kernel(CountV3Args a) {
+    __shared__ int32_t scan[1024];
+    const int t = threadIdx.x;
+    // each thread owns a contiguous run of experts; exclusive prefix of (count, non-empty) over the runs through LDS
+    const int per = (a.active + 1023) / 1024;
+    const int first = t * per, last = min(first + per, a.active);
+    int64_t sum = 0;
+    int32_t nonEmpty = 0;
+    for (int e = first; e < last; ++e) {
+        const int32_t c = a.counts != nullptr ? a.counts[e] : 0;
+        sum += c;
+        nonEmpty += c != 0 ? 1 : 0;
+    }
+    auto exclusive = [&](int32_t v) -> int32_t {
+        scan[t] = v;
+        __syncthreads();
+        for (int d = 1; d < 1024; d <<= 1) {
+            const int32_t add = t >= d ? scan[t - d] : 0;
+            __syncthreads();
+            scan[t] += add;
+            __syncthreads();
+        }
+        const int32_t r = scan[t] - v;
+        __syncthreads();
+        return r;
+    };
+    int64_t running = exclusive(static_cast<int32_t>(sum));
+    int32_t slot = exclusive(nonEmpty);
+    if (a.mode == 2) {
+        for (int i = t; i < 2 * a.kvPairs; i += 1024) a.out[i] = 0;
+        __syncthreads();
+    }
+    for (int e = first; e < last; ++e) {
+        const int32_t c = a.counts != nullptr ? a.counts[e] : 0;
+        running += c;
+        if (a.mode == 0) a.out[e] = running;
+        else if (a.mode == 1) a.out[e] = c;
+        else if (c != 0 && slot < a.kvPairs) {
+            a.out[2 * slot] = a.expertStart + e;
+            a.out[2 * slot + 1] = c;
+            ++slot;
+        }
+    }
+}
+
+// V3: expandedScale[destination] = scale[source / K] through the scatter-type map.
+__global__ void ScatterScaleKernel(const float* scale, float* expandedScale, const int32_t* rowIdx, int64_t total,
+                                   int32_t topK) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int32_t d = rowIdx[i];
+    if (d >= 0) expandedScale[d] = scale[i / topK];
+}
+
 int CeilLog2(int64_t v) {
     int b = 0;
     while ((1ll << b) < v) ++b;
@@ -296,6 +384,17 @@ class InitRoutingExecutor : public aclOpExecutor {
     int64_t tokens = 0, topK = 0, rowBytes = 0, total = 0, activeRows = 0;
     int64_t expertNum = 0, capacity = 0;
     int dropPad = 0, countFlag = 0;
+    // V3 only
+    bool v3 = false;
+    int32_t expertStart = 0, expertEnd = 0;  // active range; keys are remapped when it is not [0, expertNum)
+    bool remap = false;
+    int32_t* gatherIdxOut = nullptr;          // rowIdxType 0: the caller's index output is the gather-type map
+    int64_t* count64 = nullptr;
+    int countMode = 1;
+    int32_t kvPairs = 0;
+    const float* scale = nullptr;
+    float* expandedScale = nullptr;
+    uint64_t offRemapKeys = 0, offCounts = 0, offScatterMap = 0;
     // plan
     int passes = 1;
     int bitsPerPass[4] = {0, 0, 0, 0};
@@ -341,6 +440,11 @@ class InitRoutingExecutor : public aclOpExecutor {
         offTable = take(static_cast<uint64_t>(numSlices) * kMaxBins * 4);
         offBinBase = take(kMaxBins * 4);
         offBinTotal = take(kMaxBins * 4);
+        if (v3) {
+            offRemapKeys = remap ? take(static_cast<uint64_t>(total) * 4) : 0;
+            offCounts = take(static_cast<uint64_t>(expertNum) * 4);
+            offScatterMap = gatherIdxOut != nullptr ? take(static_cast<uint64_t>(total) * 4) : 0;
+        }
         workspaceBytes = total > 0 ? off : 0;
     }
 
@@ -353,18 +457,35 @@ class InitRoutingExecutor : public aclOpExecutor {
                                rowBytes);
         }
         GatherArgs g{x, expandedX, expandedRowIdx, rowBytes, tokens, static_cast<int32_t>(topK),
-                     dropPad ? expertNum * capacity : activeRows};
+                     dropPad ? expertNum * capacity : activeRows, scale, expandedScale};
         hipLaunchKernelGGL(GatherRowsKernel<Vec>, dim3(static_cast<unsigned>(tokens)), dim3(kGatherThreads), 0, stream,
                            g);
     }
 
     aclnnStatus Run(void* workspace, hipStream_t stream) override {
-        if (total == 0) return ACLNN_SUCCESS;
+        if (total == 0) {
+            if (v3) {  // nothing routed: the count output is still defined (all zero)
+                CountV3Args ca{nullptr, count64, expertEnd - expertStart, expertStart, countMode, kvPairs};
+                hipLaunchKernelGGL(CountV3Kernel, dim3(1), dim3(1024), 0, stream, ca);
+            }
+            return ACLNN_SUCCESS;
+        }
         char* ws = static_cast<char*>(workspace);
         const unsigned sortBlocks = static_cast<unsigned>((numSlices + kWavesPerBlock - 1) / kWavesPerBlock);
         int shift = 0;
         const int32_t* keysIn = expertIdx;
         const int32_t* payloadIn = nullptr;
+        if (v3) {
+            // expertNum counts the sort's key values here: the active experts plus, when remapping, the sentinel
+            if (remap) {
+                int32_t* keys = reinterpret_cast<int32_t*>(ws + offRemapKeys);
+                hipLaunchKernelGGL(RemapKeysKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream,
+                                   expertIdx, keys, total, expertStart, expertEnd);
+                keysIn = keys;
+            }
+            countOrCumsum = reinterpret_cast<int32_t*>(ws + offCounts);  // int32 counts of every key value
+            if (gatherIdxOut != nullptr) expandedRowIdx = reinterpret_cast<int32_t*>(ws + offScatterMap);
+        }
         for (int pass = 0; pass < passes; ++pass) {
             const bool last = pass == passes - 1;
             SortPass p{};
@@ -386,7 +507,8 @@ class InitRoutingExecutor : public aclOpExecutor {
                 co.countOrCumsum = countOrCumsum;
                 co.beforeCapacity = beforeCapacity;
             }
-            InverseMap im{last ? expandedRowIdx : nullptr, dropPad, static_cast<int32_t>(capacity)};
+            InverseMap im{last ? expandedRowIdx : nullptr, dropPad, static_cast<int32_t>(capacity),
+                          last ? gatherIdxOut : nullptr, (remap && passes == 1) ? expertEnd - expertStart : -1};
             {
                 opapi::KernelTimer timer("routing_histogram", stream);
                 hipLaunchKernelGGL(DigitHistogramKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p);
@@ -407,6 +529,14 @@ class InitRoutingExecutor : public aclOpExecutor {
             CountOutputs co{countOrCumsum, beforeCapacity, countFlag, static_cast<int32_t>(expertNum)};
             const unsigned blocks = static_cast<unsigned>((expertNum + 255) / 256);
             hipLaunchKernelGGL(CountFromSortedKernel, dim3(blocks), dim3(256), 0, stream, keysIn, total, co);
+        }
+        if (v3) {
+            CountV3Args ca{countOrCumsum, count64, expertEnd - expertStart, expertStart, countMode, kvPairs};
+            hipLaunchKernelGGL(CountV3Kernel, dim3(1), dim3(1024), 0, stream, ca);
+            if (scale != nullptr && !(rowBytes > 0 && tokens > 0)) {  // otherwise the row gather carries the scales
+                hipLaunchKernelGGL(ScatterScaleKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                                   stream, scale, expandedScale, expandedRowIdx, total, static_cast<int32_t>(topK));
+            }
         }
         if (rowBytes > 0 && tokens > 0) {
             opapi::KernelTimer timer("routing_gather", stream);
@@ -535,6 +665,138 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
 }
 
 extern "C" aclnnStatus aclnnMoeInitRoutingV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
+                                             aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
+}
+
+// ---------------------------------------------------------------------------------------------- aclnnMoeInitRoutingV3
+extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
+    const aclTensor* x, const aclTensor* expertIdx, const aclTensor* scaleOptional, const aclTensor* offsetOptional,
+    int64_t activeNum, int64_t expertCapacity, int64_t expertNum, int64_t dropPadMode, int64_t expertTokensNumType,
+    bool expertTokensNumFlag, int64_t quantMode, const aclIntArray* activeExpertRangeOptional, int64_t rowIdxType,
+    const aclTensor* expandedXOut, const aclTensor* expandedRowIdxOut, const aclTensor* expertTokensCountOrCumsumOut,
+    const aclTensor* expandedScaleOut, uint64_t* workspaceSize, aclOpExecutor** executor) {
+    using namespace opapi;
+    ClearError();
+    OPAPI_CHECK_NOTNULL(x, "x");
+    OPAPI_CHECK_NOTNULL(expertIdx, "expertIdx");
+    OPAPI_CHECK_NOTNULL(expandedXOut, "expandedXOut");
+    OPAPI_CHECK_NOTNULL(expandedRowIdxOut, "expandedRowIdxOut");
+    OPAPI_CHECK_NOTNULL(expertTokensCountOrCumsumOut, "expertTokensCountOrCumsumOut");
+    OPAPI_CHECK_NOTNULL(workspaceSize, "workspaceSize");
+    OPAPI_CHECK_NOTNULL(executor, "executor");
+    (void)expertCapacity;  // unused by the reference as well (dropless only)
+
+    constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;
+    // attributes, in the order of the reference's CheckAttr
+    int64_t expertStart = 0, expertEnd = expertNum;
+    if (activeExpertRangeOptional != nullptr) {
+        OPAPI_CHECK(activeExpertRangeOptional->values.size() == 2, kInvalid, "The dim number of expert_range should be 2.");
+        expertStart = activeExpertRangeOptional->values[0];
+        expertEnd = activeExpertRangeOptional->values[1];
+    }
+    OPAPI_CHECK(activeNum >= -1, kInvalid, "active_num should be greater than or equal to -1");
+    OPAPI_CHECK(expertNum > 0, kInvalid, "expert_num should be greater than 0");
+    OPAPI_CHECK(dropPadMode == 0, kInvalid, "drop_pad_mode currently support 0");
+    OPAPI_CHECK(expertTokensNumType >= 0 && expertTokensNumType <= 2, kInvalid,
+                "expert_tokens_num_type currently not support %lld", (long long)expertTokensNumType);
+    OPAPI_CHECK(expertTokensNumFlag, kInvalid, "expert_tokens_num_flag currently support True");
+    OPAPI_CHECK(expertStart >= 0, kInvalid, "expert_start should be greater than or equal to 0");
+    OPAPI_CHECK(expertStart < expertEnd, kInvalid, "expert_start should be less than expert_end");
+    OPAPI_CHECK(expertEnd <= expertNum, kInvalid, "expert_end should be less than or equal to %lld", (long long)expertNum);
+    OPAPI_CHECK(expertEnd <= (expertTokensNumType == 2 ? 5120 : 10240), kInvalid,
+                "expert_end should be less than or equal to %d%s", expertTokensNumType == 2 ? 5120 : 10240,
+                expertTokensNumType == 2 ? " in KEY_VALUE mode" : "");
+    OPAPI_CHECK(quantMode == -1 || quantMode == 1, kInvalid, "quant_mode currently support -1 or 1");
+    OPAPI_CHECK(quantMode == -1, kInvalid, "quant_mode 1 (dynamic quantisation) is not supported in this build");
+    OPAPI_CHECK(rowIdxType == 0 || rowIdxType == 1, kInvalid, "row_idx_type currently support 1 or 0");
+    // offset only matters to static quantisation; like the reference, accept a FLOAT tensor and ignore it
+    OPAPI_CHECK(offsetOptional == nullptr || offsetOptional->dtype == ACL_FLOAT, kInvalid, "offset must be FLOAT");
+
+    OPAPI_CHECK(x->dtype == ACL_FLOAT || x->dtype == ACL_FLOAT16 || x->dtype == ACL_BF16 || x->dtype == ACL_INT8, kInvalid,
+                "x dtype %d is not supported (FLOAT, FLOAT16, BF16, INT8)", (int)x->dtype);
+    OPAPI_CHECK(expertIdx->dtype == ACL_INT32, kInvalid, "expertIdx must be INT32");
+    OPAPI_CHECK(x->dims.size() == 2, kInvalid, "The dim number of x should be 2.");
+    OPAPI_CHECK(expertIdx->dims.size() == 2, kInvalid, "The dim number of expert_idx should be 2.");
+    OPAPI_CHECK(x->dims[0] == expertIdx->dims[0], kInvalid, "Input rows should be same.");
+    const int64_t tokens = x->dims[0], cols = x->dims[1], topK = expertIdx->dims[1];
+    const int64_t total = tokens * topK;
+    OPAPI_CHECK(total < (1ll << 31), kInvalid, "tokens * topK = %lld does not fit int32 row indices", (long long)total);
+    OPAPI_CHECK(activeNum == -1 || activeNum == total, kInvalid, "active_num currently should equal to %lld(bs*k)",
+                (long long)total);
+    const int64_t active = expertEnd - expertStart;
+    const bool remap = !(expertStart == 0 && expertEnd == expertNum);
+    OPAPI_CHECK(active + (remap ? 1 : 0) <= kMaxBins, kInvalid,
+                "this build routes at most %d active experts (%d when the range is a proper sub-range)", kMaxBins,
+                kMaxBins - 1);
+
+    if (scaleOptional != nullptr) {
+        OPAPI_CHECK(scaleOptional->dtype == ACL_FLOAT, kInvalid, "scale must be FLOAT");
+        OPAPI_CHECK(scaleOptional->dims.size() == 1, kInvalid, "The dim number of scale should be 1.");
+        OPAPI_CHECK(scaleOptional->dims[0] == tokens, kInvalid, "The first dim of scale should be %lld", (long long)tokens);
+        OPAPI_CHECK(expandedScaleOut != nullptr, ACLNN_ERR_PARAM_NULLPTR, "expandedScaleOut must not be null when scale is given");
+        OPAPI_CHECK(expandedScaleOut->dtype == ACL_FLOAT && expandedScaleOut->dims.size() == 1 &&
+                        expandedScaleOut->dims[0] == total, kInvalid, "expandedScaleOut must be FLOAT [%lld]", (long long)total);
+        OPAPI_CHECK(IsContiguous(scaleOptional) && IsContiguous(expandedScaleOut), kInvalid, "scale tensors must be contiguous");
+    }
+    OPAPI_CHECK(expandedXOut->dtype == x->dtype, kInvalid, "expandedXOut dtype must equal x dtype without quantisation");
+    OPAPI_CHECK(expandedXOut->dims.size() == 2 && expandedXOut->dims[0] == total && expandedXOut->dims[1] == cols, kInvalid,
+                "expandedXOut must be [%lld, %lld]", (long long)total, (long long)cols);
+    OPAPI_CHECK(expandedRowIdxOut->dtype == ACL_INT32 && expandedRowIdxOut->dims.size() == 1 &&
+                    expandedRowIdxOut->dims[0] == total, kInvalid, "expandedRowIdxOut must be INT32 [%lld]", (long long)total);
+    OPAPI_CHECK(expertTokensCountOrCumsumOut->dtype == ACL_INT64, kInvalid, "expertTokensCountOrCumsumOut must be INT64");
+    if (expertTokensNumType == 2) {
+        OPAPI_CHECK(expertTokensCountOrCumsumOut->dims.size() == 2 && expertTokensCountOrCumsumOut->dims[0] == expertNum &&
+                        expertTokensCountOrCumsumOut->dims[1] == 2, kInvalid,
+                    "expertTokensCountOrCumsumOut must be [%lld, 2] in KEY_VALUE mode", (long long)expertNum);
+    } else {
+        OPAPI_CHECK(expertTokensCountOrCumsumOut->dims.size() == 1 && expertTokensCountOrCumsumOut->dims[0] == active,
+                    kInvalid, "expertTokensCountOrCumsumOut must be [%lld]", (long long)active);
+    }
+    OPAPI_CHECK(IsContiguous(x) && IsContiguous(expertIdx) && IsContiguous(expandedXOut) && IsContiguous(expandedRowIdxOut) &&
+                    IsContiguous(expertTokensCountOrCumsumOut), kInvalid, "all tensors must be contiguous");
+    OPAPI_CHECK(expertTokensCountOrCumsumOut->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
+                "expertTokensCountOrCumsumOut carries no device memory");
+    if (total > 0) {
+        OPAPI_CHECK(expertIdx->data != nullptr && expandedRowIdxOut->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
+                    "expertIdx / expandedRowIdxOut carry no device memory");
+        OPAPI_CHECK(cols == 0 || (x->data != nullptr && expandedXOut->data != nullptr), ACLNN_ERR_PARAM_NULLPTR,
+                    "x / expandedXOut carry no device memory");
+        OPAPI_CHECK(scaleOptional == nullptr || (scaleOptional->data != nullptr && expandedScaleOut->data != nullptr),
+                    ACLNN_ERR_PARAM_NULLPTR, "scale / expandedScaleOut carry no device memory");
+    }
+
+    auto* ex = new (std::nothrow) InitRoutingExecutor();
+    OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
+    ex->v3 = true;
+    ex->x = DataPtr(x);
+    ex->expertIdx = reinterpret_cast<const int32_t*>(DataPtr(expertIdx));
+    ex->expandedX = DataPtr(expandedXOut);
+    if (rowIdxType == 1) ex->expandedRowIdx = reinterpret_cast<int32_t*>(DataPtr(expandedRowIdxOut));
+    else ex->gatherIdxOut = reinterpret_cast<int32_t*>(DataPtr(expandedRowIdxOut));
+    ex->count64 = reinterpret_cast<int64_t*>(DataPtr(expertTokensCountOrCumsumOut));
+    ex->countMode = static_cast<int>(expertTokensNumType);
+    // key/value pairs written: min(active + 1, expertNum), as the reference sizes its copy-out
+    ex->kvPairs = static_cast<int32_t>(active + 1 < expertNum ? active + 1 : expertNum);
+    ex->scale = scaleOptional != nullptr ? reinterpret_cast<const float*>(DataPtr(scaleOptional)) : nullptr;
+    ex->expandedScale = scaleOptional != nullptr ? reinterpret_cast<float*>(DataPtr(expandedScaleOut)) : nullptr;
+    ex->expertStart = static_cast<int32_t>(expertStart);
+    ex->expertEnd = static_cast<int32_t>(expertEnd);
+    ex->remap = remap;
+    ex->tokens = tokens;
+    ex->topK = topK;
+    ex->rowBytes = cols * ElemSize(x->dtype);
+    ex->total = total;
+    ex->activeRows = total;
+    ex->expertNum = active + (remap ? 1 : 0);  // key values the sort sees
+    ex->countFlag = 2;                          // the sort emits plain int32 counts; CountV3Kernel shapes the output
+    ex->Plan();
+    *workspaceSize = ex->workspaceBytes;
+    *executor = ex;
+    return ACLNN_SUCCESS;
+}
+
+extern "C" aclnnStatus aclnnMoeInitRoutingV3(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
                                              aclrtStream stream) {
     return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
 }

@@ -1,15 +1,17 @@
 """The quantized MoE expert FFN as a chain of the four aclnn operators (the caller side of the path).
 
-    aclnnMoeInitRoutingV2 -> aclnnGroupedMatmulSwigluQuant -> aclnnGroupedMatmulV4 -> aclnnMoeFinalizeRoutingV2
+    aclnnMoeInitRoutingV3 -> aclnnGroupedMatmulSwigluQuant -> aclnnGroupedMatmulV4 -> aclnnMoeFinalizeRoutingV2
 
 The reference has no in-repo code that chains them; real callers (torch_npu, vLLM-Ascend) do what ``forward`` does.
 Glue between the operators:
-  * activations arrive already quantized per token (int8 rows + fp32 scale); the rows are routed with the INT8
-    extension of MoeInitRoutingV2 and the per-token scales are routed by a second MoeInitRoutingV2 call on the
-    [T, 1] fp32 scale column (a row gather commutes with per-row quantization bit-exactly);
-  * routing emits an int32 cumsum; both GEMM operators of this build accept it directly;
-  * MoeFinalizeRoutingV2 is called with dropPadMode 2 because MoeInitRoutingV2 emits the row arrangement
-    (expandedRowIdx[n*K + k]).
+  * activations arrive already quantized per token (int8 rows + fp32 scale); one MoeInitRoutingV3 call (quantMode -1,
+    INT8 x as this build's extension) routes the rows and carries the per-token scales along as expandedScale
+    (a row gather commutes with per-row quantization bit-exactly);
+  * routing emits the int64 cumsum (expertTokensNumType 0) both GEMM operators take as groupList;
+  * MoeFinalizeRoutingV2 is called with dropPadMode 2 because the scatter-type index (rowIdxType 1) is the row
+    arrangement expandedRowIdx[n*K + k] = destination.
+``routing="v2"`` keeps the older chain: MoeInitRoutingV2 on the rows plus a second MoeInitRoutingV2 call on the
+[T, 1] scale column, int32 cumsum.
 """
 import torch
 
@@ -27,7 +29,9 @@ class MoeFfnW8A8:
     The operators see the reference layout [E, K, N] through transposed views of this storage.
     """
 
-    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16):
+    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v3"):
+        assert routing in ("v2", "v3")
+        self.routing = routing
         assert w13.dtype == torch.int8 and w2.dtype == torch.int8
         self.w13_view = w13.transpose(1, 2)  # [E, H, 2I]
         self.w2_view = w2.transpose(1, 2)    # [E, I, H]
@@ -46,8 +50,8 @@ class MoeFfnW8A8:
         dev, M, H, I, E = self.device, T * K, self.hidden, self.inter, self.num_experts
         self.expanded_x = torch.empty((M, H), dtype=torch.int8, device=dev)
         self.expanded_row_idx = torch.empty((M,), dtype=torch.int32, device=dev)
-        self.cumsum = torch.empty((E,), dtype=torch.int32, device=dev)
-        self.expanded_scale = torch.empty((M, 1), dtype=torch.float32, device=dev)
+        self.cumsum = torch.empty((E,), dtype=torch.int64 if self.routing == "v3" else torch.int32, device=dev)
+        self.expanded_scale = torch.empty((M,), dtype=torch.float32, device=dev)
         self.row_idx_scratch = torch.empty((M,), dtype=torch.int32, device=dev)
         self.h = torch.empty((M, I), dtype=torch.int8, device=dev)
         self.h_scale = torch.empty((M,), dtype=torch.float32, device=dev)
@@ -62,14 +66,20 @@ class MoeFfnW8A8:
         T, K = topk_idx.shape
         self._buffers(T, K)
         E = self.num_experts
-        aclnn.moe_init_routing_v2(xq, topk_idx, 0, 0, E, 0, 1, False,
-                                  out=(self.expanded_x, self.expanded_row_idx, self.cumsum, None),
-                                  workspace=self.workspace)
-        aclnn.moe_init_routing_v2(x_scale.view(T, 1), topk_idx, 0, 0, E, 0, 0, False,
-                                  out=(self.expanded_scale, self.row_idx_scratch, None, None),
-                                  workspace=self.workspace)
+        if self.routing == "v3":
+            aclnn.moe_init_routing_v3(xq, topk_idx, x_scale, expert_num=E, expert_tokens_num_type=0, quant_mode=-1,
+                                      row_idx_type=1,
+                                      out=(self.expanded_x, self.expanded_row_idx, self.cumsum, self.expanded_scale),
+                                      workspace=self.workspace)
+        else:
+            aclnn.moe_init_routing_v2(xq, topk_idx, 0, 0, E, 0, 1, False,
+                                      out=(self.expanded_x, self.expanded_row_idx, self.cumsum, None),
+                                      workspace=self.workspace)
+            aclnn.moe_init_routing_v2(x_scale.view(T, 1), topk_idx, 0, 0, E, 0, 0, False,
+                                      out=(self.expanded_scale.view(T * K, 1), self.row_idx_scratch, None, None),
+                                      workspace=self.workspace)
         aclnn.grouped_matmul_swiglu_quant(self.expanded_x, self.w13_view, self.cumsum, self.w13_scale,
-                                          self.expanded_scale.view(T * K), out=(self.h, self.h_scale),
+                                          self.expanded_scale, out=(self.h, self.h_scale),
                                           workspace=self.workspace)
         aclnn.grouped_matmul_v4([self.h], [self.w2_view], scale=[self.w2_scale], per_token_scale=[self.h_scale],
                                 group_list=self.cumsum, split_item=3, group_type=0, group_list_type=0, act_type=0,

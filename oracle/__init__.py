@@ -128,6 +128,31 @@ def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_n
     return ex, idx, cnt, bef
 
 
+def moe_init_routing_v3(x, expert_idx, scale=None, expert_num=0, expert_range=None, count_mode=1, row_idx_type=1):
+    """Dropless, unquantised MoeInitRoutingV3.  Returns (expandedX, idx int32 [M], counts int64, expandedScale or None).
+    Output rows that no routed row lands on are zero."""
+    x = np.ascontiguousarray(x)
+    T = x.shape[0]
+    row_bytes = x.strides[0] if x.ndim == 2 and x.shape[1] > 0 else 0
+    idx = _c(expert_idx, np.int32)
+    K = idx.shape[1]
+    M = T * K
+    start, end = (0, expert_num) if expert_range is None else expert_range
+    ex = np.zeros((M,) + x.shape[1:], x.dtype)
+    out_idx = np.zeros((M,), np.int32)
+    if count_mode == 2:
+        counts = np.zeros((expert_num, 2), np.int64)
+    else:
+        counts = np.zeros((end - start,), np.int64)
+    sc = None if scale is None else _c(scale, np.float32)
+    ex_scale = None if scale is None else np.zeros((M,), np.float32)
+    lib().oracle_moe_init_routing_v3(
+        _p(x), ctypes.c_int64(row_bytes), _p(idx), _p(sc), ctypes.c_int64(T), ctypes.c_int64(K), ctypes.c_int64(expert_num),
+        ctypes.c_int64(start), ctypes.c_int64(end), ctypes.c_int64(count_mode), ctypes.c_int64(row_idx_type), _p(ex),
+        _p(out_idx), _p(counts), _p(ex_scale))
+    return ex, out_idx, counts, ex_scale
+
+
 # ----------------------------------------------------------------------------------------------- GEMMs
 def _gemm_common(x, w, w_trans, group_list, rows):
     x = _c(x, np.int8)

@@ -185,6 +185,51 @@ ORACLE_API int oracle_moe_init_routing_v2(const void* x, int64_t rowBytes, const
     return 0;
 }
 
+/* MoeInitRoutingV3, dropless, no quantisation (moe/moe_init_routing_v3/README.md:12-66;
+ * op_kernel/moe_v3_gather_out.h:213-231 row and scale gather; op_kernel/moe_v3_expert_tokens_count.h:254-269 counts).
+ * Rows whose expert lies in [start, end) are sorted (stable) by expert and packed from destination 0; the others are
+ * dropped.  rowIdxType 1: idx[source] = destination (-1 when dropped; the reference leaves those uninitialised);
+ * rowIdxType 0: idx[destination] = source for the packed rows, -1 behind them.
+ * countMode 0 cumsum, 1 count (int64 [end-start]); 2 key/value pairs of the non-empty experts, zero-filled, written
+ * for min(end-start+1, expertNum) pairs.  Untouched output rows keep their previous contents. */
+ORACLE_API int oracle_moe_init_routing_v3(const void* x, int64_t rowBytes, const int32_t* expertIdx, const float* scale,
+                                          int64_t T, int64_t K, int64_t expertNum, int64_t start, int64_t end,
+                                          int64_t countMode, int64_t rowIdxType, void* expandedX, int32_t* idxOut,
+                                          int64_t* counts, float* expandedScale) {
+    const int64_t M = T * K, active = end - start;
+    int64_t* hist = (int64_t*)calloc((size_t)active + 1, sizeof(int64_t));
+    for (int64_t i = 0; i < M; i++) {
+        const int64_t e = expertIdx[i];
+        if (e >= start && e < end) hist[e - start + 1]++;
+    }
+    if (countMode == 2) {
+        const int64_t pairs = (active + 1 < expertNum) ? active + 1 : expertNum;
+        memset(counts, 0, sizeof(int64_t) * 2 * (size_t)pairs);
+        int64_t slot = 0;
+        for (int64_t e = 0; e < active; e++) {
+            if (hist[e + 1] != 0 && slot < pairs) { counts[2 * slot] = start + e; counts[2 * slot + 1] = hist[e + 1]; slot++; }
+        }
+    }
+    int64_t run = 0;
+    for (int64_t e = 0; e < active; e++) {
+        run += hist[e + 1];
+        if (countMode == 0) counts[e] = run;
+        if (countMode == 1) counts[e] = hist[e + 1];
+    }
+    for (int64_t e = 0; e < active; e++) hist[e + 1] += hist[e];   /* hist[e] = first destination of expert start+e */
+    for (int64_t i = 0; i < M; i++) idxOut[i] = -1;
+    for (int64_t i = 0; i < M; i++) {                                /* ascending source index => stable */
+        const int64_t e = expertIdx[i];
+        if (e < start || e >= end) continue;
+        const int64_t d = hist[e - start]++;
+        if (rowIdxType == 1) idxOut[i] = (int32_t)d; else idxOut[d] = (int32_t)i;
+        if (expandedX && rowBytes > 0) memcpy((char*)expandedX + d * rowBytes, (const char*)x + (i / K) * rowBytes, (size_t)rowBytes);
+        if (scale && expandedScale) expandedScale[d] = scale[i / K];
+    }
+    free(hist);
+    return 0;
+}
+
 /* ------------------------------------------------------------------------------------------------ grouped GEMM */
 
 /* Group boundaries from groupList: type 0 = inclusive cumsum, type 1 = per-group counts (grouped_matmul_utils.h:243-257). */

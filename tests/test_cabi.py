@@ -30,6 +30,7 @@ def _declared_symbols():
 def test_headers_declare_the_expected_entry_points():
     names = _declared_symbols()
     for required in ["aclnnMoeInitRoutingV2GetWorkspaceSize", "aclnnMoeInitRoutingV2",
+                     "aclnnMoeInitRoutingV3GetWorkspaceSize", "aclnnMoeInitRoutingV3",
                      "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize", "aclnnGroupedMatmulSwigluQuant",
                      "aclnnGroupedMatmulV4GetWorkspaceSize", "aclnnGroupedMatmulV4",
                      "aclnnGroupedMatmulV5GetWorkspaceSize", "aclnnGroupedMatmulV5",
@@ -123,6 +124,69 @@ def test_routing_null_and_rank_checks(aclnn):
     args[0] = x3.h
     code, msg = _status(aclnn, "aclnnMoeInitRoutingV2", args)
     assert code == INVALID and "dim number of x should be 2" in msg
+
+
+# ------------------------------------------------------------------------------------------------ routing V3
+def _routing_v3_args(aclnn, T_=8, K=2, H=16, E=4, rng=None, num_type=1, flag=True, quant=-1, row_idx_type=1, active=-1,
+                     mode=0, x_dtype=I8, with_scale=True, **over):
+    x = T(aclnn, (T_, H), x_dtype)
+    idx = T(aclnn, (T_, K), I32)
+    scale = T(aclnn, over.get("scale_shape", (T_,)), F32) if with_scale else None
+    start, end = (0, E) if rng is None else rng[:2]
+    ex = T(aclnn, over.get("ex_shape", (T_ * K, H)), over.get("ex_dtype", x_dtype))
+    ri = T(aclnn, over.get("ri_shape", (T_ * K,)), I32)
+    cnt = T(aclnn, over.get("cnt_shape", (E, 2) if num_type == 2 else (max(end - start, 0),)), over.get("cnt_dtype", I64))
+    es = T(aclnn, (T_ * K,), F32) if with_scale else None
+    arr = None if rng is None else aclnn.lib().aclCreateIntArray((ctypes.c_int64 * len(rng))(*rng), len(rng))
+    return [x.h, idx.h, scale.h if scale else None, None, active, 0, E, mode, num_type, flag, quant, arr, row_idx_type,
+            ex.h, ri.h, cnt.h, es.h if es else None]
+
+
+def test_routing_v3_valid(aclnn):
+    for kw in [dict(), dict(num_type=0), dict(num_type=2), dict(rng=(1, 3)), dict(row_idx_type=0), dict(active=16),
+               dict(x_dtype=BF16, with_scale=False), dict(T_=0), dict(E=2048), dict(E=4096, rng=(100, 2147))]:
+        code, ws = _status(aclnn, "aclnnMoeInitRoutingV3", _routing_v3_args(aclnn, **kw))
+        assert code == 0, (kw, ws)
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    # attribute rules and messages of moe/moe_init_routing_v3/op_host/moe_init_routing_v3_tiling.cpp:233-352
+    (dict(active=-2), "active_num should be greater than or equal to -1"),
+    (dict(active=5), "active_num currently should equal to 16"),
+    (dict(E=0, cnt_shape=(1,)), "expert_num should be greater than 0"),
+    (dict(mode=1), "drop_pad_mode currently support 0"),
+    (dict(num_type=3), "expert_tokens_num_type currently not support 3"),
+    (dict(flag=False), "expert_tokens_num_flag currently support True"),
+    (dict(rng=(-1, 3)), "expert_start should be greater than or equal to 0"),
+    (dict(rng=(3, 3)), "expert_start should be less than expert_end"),
+    (dict(rng=(0, 5)), "expert_end should be less than or equal to 4"),
+    (dict(rng=(0, 1, 2)), "dim number of expert_range should be 2"),
+    (dict(quant=0), "quant_mode currently support -1 or 1"),
+    (dict(quant=1), "not supported in this build"),
+    (dict(row_idx_type=2), "row_idx_type currently support 1 or 0"),
+    (dict(scale_shape=(9,)), "first dim of scale should be 8"),
+    (dict(scale_shape=(8, 1)), "dim number of scale should be 1"),
+    (dict(ex_shape=(15, 16)), "expandedXOut must be [16, 16]"),
+    (dict(ex_dtype=F32), "expandedXOut dtype"),
+    (dict(ri_shape=(15,)), "expandedRowIdxOut must be INT32 [16]"),
+    (dict(cnt_dtype=I32), "must be INT64"),
+    (dict(cnt_shape=(5,)), "expertTokensCountOrCumsumOut must be [4]"),
+    (dict(num_type=2, cnt_shape=(4,)), "[4, 2] in KEY_VALUE mode"),
+    (dict(E=4096), "at most 2048 active experts"),
+])
+def test_routing_v3_invalid(aclnn, kw, fragment):
+    code, msg = _status(aclnn, "aclnnMoeInitRoutingV3", _routing_v3_args(aclnn, **kw))
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_routing_v3_nulls(aclnn):
+    for pos in (0, 1, 13, 14, 15):
+        args = _routing_v3_args(aclnn)
+        args[pos] = None
+        assert _status(aclnn, "aclnnMoeInitRoutingV3", args)[0] == NULLPTR, pos
+    args = _routing_v3_args(aclnn)
+    args[16] = None                      # scale given, no place for the routed scales
+    assert _status(aclnn, "aclnnMoeInitRoutingV3", args)[0] == NULLPTR
 
 
 # ------------------------------------------------------------------------------------------------ SwiGLU quant

@@ -74,3 +74,18 @@ def test_decode_config_sampled(pkg, oracle, dev):
     ref = oracle.moe_finalize_routing_v2(y, row_idx, scales=wgt, drop_pad_mode=2, dtype=oracle.DT_BF16,
                                          scale_dtype=oracle.DT_F32)
     assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+
+
+def test_v2_and_v3_routing_chains_agree(pkg, dev):
+    """The chain routed by one MoeInitRoutingV3 call equals the chain routed by two MoeInitRoutingV2 calls, bit for bit."""
+    cfg = pkg.synth.config(0)
+    idx, wgt = pkg.synth.make_routing(cfg, seed=0)
+    xq, xs = pkg.synth.make_activations(cfg, seed=0)
+    w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=0)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    outs = []
+    for routing in ("v3", "v2"):
+        ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, routing=routing)
+        outs.append(ffn.forward(t(xq), t(xs), t(idx), t(wgt)).clone())
+        torch.cuda.synchronize()
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))

@@ -117,3 +117,74 @@ def test_empty_inputs(aclnn, dev):
     ex, ri, _, _ = aclnn.moe_init_routing_v2(x, idx, expert_num=4)
     torch.cuda.synchronize()
     assert ex.shape == (0, 16) and ri.shape == (0,)
+
+
+# ------------------------------------------------------------------------------------------------ MoeInitRoutingV3
+def _run_v3(aclnn, dev, x, idx, scale, **kw):
+    outs = aclnn.moe_init_routing_v3(torch.from_numpy(x).to(dev), torch.from_numpy(idx).to(dev),
+                                     None if scale is None else torch.from_numpy(scale).to(dev), **kw)
+    torch.cuda.synchronize()
+    return [None if o is None else o.cpu().numpy() for o in outs]
+
+
+V3_CASES = [  # T, K, E, H, dtype, expert range
+    (1, 1, 1, 1, np.float32, None),
+    (3, 4, 256, 2, np.float32, (0, 4)),          # the reference example's shape
+    (7, 3, 5, 30, np.float16, (1, 4)),
+    (64, 8, 128, 4096, np.int8, None),           # decode shape
+    (64, 8, 256, 512, np.int8, (32, 64)),        # one expert-parallel rank's share of 256 experts
+    (333, 5, 100, 7, np.float32, (99, 100)),     # a single active expert, odd row bytes
+    (1000, 4, 33, 18, np.int8, (0, 32)),
+    (4096, 8, 256, 512, np.int8, None),          # DeepSeek-V3 routing shape
+    (2048, 6, 4000, 8, np.float32, (1000, 3047)),  # 2047 active experts + the sentinel: the full 11-bit digit
+    (2048, 6, 2048, 8, np.float32, None),
+]
+
+
+@pytest.mark.parametrize("T,K,E,H,dtype,rng_", V3_CASES)
+def test_v3_bit_exact(aclnn, oracle, dev, T, K, E, H, dtype, rng_):
+    rng = np.random.default_rng(T * 11 + K)
+    x = (rng.standard_normal((T, H)) * 50).astype(dtype)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    scale = rng.random(T).astype(np.float32)
+    for mode in (0, 1, 2):
+        for row_idx_type in (1, 0):
+            ex, ri, cnt, es = _run_v3(aclnn, dev, x, idx, scale, expert_num=E, expert_tokens_num_type=mode,
+                                      active_expert_range=rng_, row_idx_type=row_idx_type)
+            ex_r, ri_r, cnt_r, es_r = oracle.moe_init_routing_v3(x, idx, scale, E, rng_, mode, row_idx_type)
+            assert np.array_equal(ri, ri_r), (mode, row_idx_type)
+            assert np.array_equal(cnt, cnt_r), (mode, row_idx_type)
+            assert np.array_equal(ex.view(np.uint8), ex_r.view(np.uint8))
+            assert np.array_equal(es, es_r)
+
+
+def test_v3_without_scale_and_empty_input(aclnn, oracle, dev):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((50, 12)).astype(np.float32)
+    idx = rng.integers(0, 9, (50, 3)).astype(np.int32)
+    ex, ri, cnt, es = _run_v3(aclnn, dev, x, idx, None, expert_num=9, active_expert_range=(2, 7))
+    ex_r, ri_r, cnt_r, _ = oracle.moe_init_routing_v3(x, idx, None, 9, (2, 7), 1, 1)
+    assert es is None and np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r) and np.array_equal(ex, ex_r)
+    # no tokens: the count output is still written
+    for mode, shape in ((0, (5,)), (1, (5,)), (2, (9, 2))):
+        counts = torch.full(shape, 77, dtype=torch.int64, device=dev)
+        out = (torch.empty((0, 12), device=dev), torch.empty((0,), dtype=torch.int32, device=dev), counts, None)
+        aclnn.moe_init_routing_v3(torch.empty((0, 12), device=dev), torch.empty((0, 3), dtype=torch.int32, device=dev),
+                                  None, expert_num=9, expert_tokens_num_type=mode, active_expert_range=(2, 7), out=out)
+        torch.cuda.synchronize()
+        got = counts.cpu().numpy()
+        if mode == 2:   # min(active + 1, expertNum) = 6 pairs are written, the rest of the buffer is the caller's
+            assert not got[:6].any() and (got[6:] == 77).all()
+        else:
+            assert not got.any()
+
+
+def test_v3_skewed_routing_matches_v2(pkg, aclnn, dev):
+    """Zipf-skewed load, whole range: V3's scatter-type index, cumsum and rows equal V2's (int64 instead of int32)."""
+    cfg = pkg.synth.config(4)
+    idx, _ = pkg.synth.make_routing(cfg, seed=4)
+    x = np.arange(cfg.tokens * 16, dtype=np.int32).reshape(cfg.tokens, 16).view(np.float32)
+    ex2, ri2, cum2, _ = _run(aclnn, dev, x, idx, expert_num=cfg.experts, expert_tokens_count_or_cumsum_flag=1)
+    ex3, ri3, cum3, _ = _run_v3(aclnn, dev, x, idx, None, expert_num=cfg.experts, expert_tokens_num_type=0)
+    assert np.array_equal(ri2, ri3) and np.array_equal(cum2.astype(np.int64), cum3)
+    assert np.array_equal(ex2.view(np.uint32), ex3.view(np.uint32))

@@ -103,3 +103,71 @@ def test_unknown_expert_range_sorts_signed(oracle):
     ref = np.empty(600, np.int32)
     ref[order] = np.arange(600, dtype=np.int32)
     assert np.array_equal(ri, ref)
+
+
+# ------------------------------------------------------------------------------------------------ MoeInitRoutingV3
+def _numpy_v3(x, idx, scale, start, end):
+    """Stable argsort of the in-range flat positions: the sort + filter the reference kernels implement
+    (moe/moe_init_routing_v3/README.md:12-66)."""
+    T, K = idx.shape
+    flat = idx.reshape(-1)
+    keep = np.nonzero((flat >= start) & (flat < end))[0]
+    order = keep[np.argsort(flat[keep], kind="stable")]
+    hist = np.bincount(flat[keep] - start, minlength=end - start)
+    return order, hist
+
+
+@pytest.mark.parametrize("T,K,E,H,rng_", [(1, 1, 1, 1, None), (7, 3, 5, 4, (1, 4)), (64, 8, 256, 16, (32, 64)),
+                                          (333, 2, 8, 7, None), (500, 4, 33, 3, (0, 1)), (40, 2, 16, 2, (15, 16))])
+def test_v3_matches_numpy(oracle, T, K, E, H, rng_):
+    rng = np.random.default_rng(T * 17 + K)
+    x = rng.integers(-128, 128, (T, H)).astype(np.int8)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    scale = rng.random(T).astype(np.float32)
+    start, end = (0, E) if rng_ is None else rng_
+    order, hist = _numpy_v3(x, idx, scale, start, end)
+    n = len(order)
+    for mode in (0, 1, 2):
+        for row_idx_type in (0, 1):
+            ex, ri, cnt, es = oracle.moe_init_routing_v3(x, idx, scale, E, rng_, mode, row_idx_type)
+            assert np.array_equal(ex[:n], x[order // K]) and not ex[n:].any()
+            assert np.array_equal(es[:n], scale[order // K])
+            if row_idx_type == 0:
+                assert np.array_equal(ri[:n], order) and (ri[n:] == -1).all()
+            else:
+                inverse = np.full(T * K, -1, np.int32)
+                inverse[order] = np.arange(n)
+                assert np.array_equal(ri, inverse)
+            if mode == 0:
+                assert np.array_equal(cnt, np.cumsum(hist))
+            elif mode == 1:
+                assert np.array_equal(cnt, hist)
+            else:
+                nz = np.nonzero(hist)[0]
+                assert cnt.shape == (E, 2)
+                assert np.array_equal(cnt[:len(nz), 0], nz + start) and np.array_equal(cnt[:len(nz), 1], hist[nz])
+                assert not cnt[len(nz):].any()
+
+
+def test_v3_full_range_equals_v2(oracle):
+    """With the whole expert range active V3 is V2's dropless mode with int64 counts."""
+    rng = np.random.default_rng(5)
+    T, K, E, H = 200, 4, 24, 6
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    ex2, ri2, cum2, _ = oracle.moe_init_routing_v2(x, idx, expert_num=E, count_flag=1)
+    ex3, ri3, cum3, _ = oracle.moe_init_routing_v3(x, idx, None, E, None, 0, 1)
+    assert np.array_equal(ex2, ex3) and np.array_equal(ri2, ri3) and np.array_equal(cum2.astype(np.int64), cum3)
+
+
+def test_v3_reference_example_literal(oracle):
+    """Inputs of moe/moe_init_routing_v3/examples/test_aclnn_moe_init_routing_v3.cpp:123-125 (range [0, 4), count
+    mode); the expected values follow from the operator's definition by hand."""
+    x = np.array([[0.1, 0.1], [0.2, 0.2], [0.3, 0.3]], np.float32)
+    idx = np.array([[1, 2, 0, 3], [0, 2, 1, 3], [0, 1, 3, 2]], np.int32)
+    scale = np.array([0.3423, 0.1652, 0.2652], np.float32)
+    ex, ri, cnt, es = oracle.moe_init_routing_v3(x, idx, scale, 256, (0, 4), 1, 1)
+    assert ri.tolist() == [3, 6, 0, 9, 1, 7, 4, 10, 2, 5, 11, 8]
+    assert cnt.tolist() == [3, 3, 3, 3]
+    assert np.array_equal(ex[:, 0], np.array([0.1, 0.2, 0.3, 0.1, 0.2, 0.3, 0.1, 0.2, 0.3, 0.1, 0.2, 0.3], np.float32))
+    assert np.array_equal(es, scale[[0, 1, 2] * 4])
