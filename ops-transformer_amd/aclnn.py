@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.environ.get("OPAPI_LIBRARY_PATH") or os.path.join(_HERE, "lib", "libcust_opapi.so")
 
-ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32, ACL_INT64, ACL_BF16 = 0, 1, 2, 3, 9, 27
+ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32, ACL_INT64, ACL_BOOL, ACL_BF16 = 0, 1, 2, 3, 9, 12, 27
 ACL_FORMAT_ND = 2
 
 ACLNN_SUCCESS = 0
@@ -29,6 +29,7 @@ _DTYPE_CODE = {
     torch.int32: ACL_INT32,
     torch.int64: ACL_INT64,
     torch.bfloat16: ACL_BF16,
+    torch.bool: ACL_BOOL,
 }
 
 
@@ -54,6 +55,8 @@ _VPP = ctypes.POINTER(ctypes.c_void_p)
 _PHASE1_SIGNATURES = {
     "aclnnMoeInitRoutingV2GetWorkspaceSize":
         [_VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize":
+        [_VP, _VP, _I64, _I64, ctypes.c_bool, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnMoeInitRoutingV3GetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _I64, _VP, _I64, _VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize":
@@ -65,7 +68,7 @@ _PHASE1_SIGNATURES = {
     "aclnnMoeFinalizeRoutingV2GetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _U64P, _VPP],
 }
-_PHASE2 = ["aclnnMoeInitRoutingV2", "aclnnMoeInitRoutingV3", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
+_PHASE2 = ["aclnnMoeGatingTopKSoftmaxV2", "aclnnMoeInitRoutingV2", "aclnnMoeInitRoutingV3", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
            "aclnnMoeFinalizeRoutingV2"]
 
 
@@ -255,6 +258,25 @@ def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_n
     finally:
         h.close()
     return expanded_x, expanded_row_idx, count_out, before_out
+
+
+def moe_gating_top_k_softmax_v2(x, k, renorm=0, finished=None, output_softmax=False, out=None):
+    """aclnnMoeGatingTopKSoftmaxV2.  Returns (y [..., k] in x's dtype, expertIdx int32 [..., k], softmax fp32 or None)."""
+    dev = x.device
+    lead = tuple(x.shape[:-1])
+    if out is not None:
+        y, idx, sm = out
+    else:
+        y = torch.empty(lead + (k,), dtype=x.dtype, device=dev)
+        idx = torch.empty(lead + (k,), dtype=torch.int32, device=dev)
+        sm = torch.empty(tuple(x.shape), dtype=torch.float32, device=dev) if (output_softmax and renorm == 0) else None
+    h = _Handles()
+    try:
+        args = [h.tensor(x), h.tensor(finished), k, renorm, bool(output_softmax), h.tensor(y), h.tensor(idx), h.tensor(sm)]
+        _run_two_phase("aclnnMoeGatingTopKSoftmaxV2", args, dev, None)
+    finally:
+        h.close()
+    return y, idx, sm
 
 
 def moe_init_routing_v3(x, expert_idx, scale=None, expert_num=0, expert_tokens_num_type=1, quant_mode=-1,

@@ -20,6 +20,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libcust_opapi.so")
 
 SOURCES = [
     "acl_runtime.cpp",
+    "moe_gating_top_k_softmax_v2.hip",
     "moe_init_routing.hip",
     "grouped_gemm_i8.hip",
     "grouped_matmul_swiglu_quant.hip",

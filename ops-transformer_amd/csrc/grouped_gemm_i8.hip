@@ -213,13 +213,6 @@ __device__ __forceinline__ float LoadScale(const void* p, int64_t i, int dtype) 
     return __uint_as_float(static_cast<uint32_t>(raw) << 16);
 }
 
-__device__ __forceinline__ uint16_t ToBf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
-}
-
 // Epilogue of one tile.  acc[mi][ni][v] is C[row, col] with row = waveRow0 + 32*mi + 8*(v/4) + 4*lhi + (v%4); the wave
 // owns column blocks ni = 0, 1, lane l32 inside each (plain: 64*waveN + 32*ni; kSwiglu: S column 32*waveN and its partner).
 // Only the first mySub accumulator tiles of the wave are real.  ldsRowScale holds the tile's per-row scales.
@@ -475,22 +468,6 @@ __device__ __forceinline__ int LdsOffset(int row, int chunk) {
     return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4);
 }
 
-// 16 bytes per lane from (uniform base + 32-bit lane offset) straight into LDS at ldsDst + lane * 16.  The compiler does
-// not see this as a memory instruction: completion is awaited with WaitVmcnt below.
-__device__ __forceinline__ void DmaToLds16(const char* base, uint32_t laneOffset, char* ldsDst) {
-    typedef __attribute__((address_space(3))) char* LdsPtr;  // the 32-bit LDS address of a generic pointer into LDS
-    const uint32_t m0 = static_cast<uint32_t>(
-        __builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(reinterpret_cast<size_t>((LdsPtr)ldsDst)))));
-    // The base is wave-uniform by construction; readfirstlane makes the compiler keep it in scalar registers.
-    // readfirstlane returns a signed int: each half is widened through uint32_t so that a low word with its top bit
-    // set cannot sign-extend into the high word.
-    const uint64_t b = reinterpret_cast<uint64_t>(base);
-    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(b))));
-    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(b >> 32))));
-    const uint64_t sbase = static_cast<uint64_t>(lo) | (static_cast<uint64_t>(hi) << 32);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(laneOffset), "s"(sbase) : "memory");
-}
-
 // A wave-uniform pointer, forced into scalar registers.
 __device__ __forceinline__ const char* UniformPtr(const char* p) {
     const uint64_t b = reinterpret_cast<uint64_t>(p);
@@ -506,7 +483,9 @@ __device__ __forceinline__ uint32_t LdsAddress(const char* p) {
         __builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(reinterpret_cast<size_t>((LdsPtr)p)))));
 }
 
-// DmaToLds16 with the destination given as a 32-bit LDS address.
+// 16 bytes per lane from (uniform base + 32-bit lane offset) straight into LDS at ldsAddr + lane * 16 (ldsAddr is the
+// 32-bit LDS address, see LdsAddress).  The compiler does not see this as a memory instruction: completion is awaited
+// with WaitVmcnt below.
 __device__ __forceinline__ void DmaToLdsAddr16(const char* base, uint32_t laneOffset, uint32_t ldsAddr) {
     const uint32_t m0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(ldsAddr)));
     const char* const sbase = UniformPtr(base);

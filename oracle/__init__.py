@@ -96,6 +96,36 @@ def from_f32(a, dtype_code):
     return f32_to_f16_bits(a) if dtype_code == DT_F16 else f32_to_bf16_bits(a)
 
 
+# ----------------------------------------------------------------------------------------------- gating
+def f32_to_f16_bits_away(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, np.uint16)
+    lib().oracle_f32_to_f16_away(_p(a), _p(out), ctypes.c_int64(a.size))
+    return out
+
+
+def f32_to_bf16_bits_away(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, np.uint16)
+    lib().oracle_f32_to_bf16_away(_p(a), _p(out), ctypes.c_int64(a.size))
+    return out
+
+
+def moe_gating_top_k_softmax_v2(x, k, renorm=0, finished=None, dtype=DT_F32, want_softmax=False):
+    """x: fp32 array, or uint16 bit patterns for DT_F16 / DT_BF16, shape [..., cols].
+    Returns (y in x's representation [..., k], expertIdx int32 [..., k], softmax fp32 [..., cols] or None)."""
+    x = _c(x)
+    cols = x.shape[-1]
+    rows = x.size // cols
+    y = np.empty(x.shape[:-1] + (k,), x.dtype)
+    idx = np.empty(x.shape[:-1] + (k,), np.int32)
+    sm = np.empty(x.shape, np.float32) if (want_softmax and renorm == 0) else None
+    fin = None if finished is None else _c(finished, np.uint8)
+    lib().oracle_moe_gating_top_k_softmax_v2(_p(x), ctypes.c_int(dtype), _p(fin), ctypes.c_int64(rows), ctypes.c_int64(cols),
+                                             ctypes.c_int64(k), ctypes.c_int64(renorm), _p(y), _p(idx), _p(sm))
+    return y, idx, sm
+
+
 # ----------------------------------------------------------------------------------------------- routing
 def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_num=0, drop_pad_mode=0,
                         count_flag=0, before_capacity_flag=False):

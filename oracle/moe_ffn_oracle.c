@@ -105,6 +105,86 @@ static inline void store_from_f32(void* p, int64_t i, int dt, float v) {
     else ((uint16_t*)p)[i] = f32_to_bf16(v);
 }
 
+/* ------------------------------------------------------------------------------------------------ gating */
+
+/* fp32 -> 16-bit with ties away from zero (Ascend C RoundMode::CAST_ROUND), done on the magnitude bits. */
+static inline uint16_t f32_to_bf16_away(float f) {
+    uint32_t u = f2u(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    return (uint16_t)((u + 0x8000u) >> 16);
+}
+static inline uint16_t f32_to_f16_away(float f) {
+    const uint32_t u = f2u(f), sign = (u >> 16) & 0x8000u, mag = u & 0x7fffffffu;
+    if (mag > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+    if (mag >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);            /* >= 65520: beyond the largest half */
+    const int32_t e = (int32_t)(mag >> 23) - 127;
+    if (e < -25) return (uint16_t)sign;                                   /* below half of the smallest subnormal */
+    uint32_t m = (mag & 0x7fffffu) | 0x800000u;                           /* 24-bit significand, value = m * 2^(e-23) */
+    /* target unit: 2^-24 for subnormals (e < -14), 2^(e-10) for normals */
+    const int shift = e < -14 ? (-24 - (e - 23)) : 13;                     /* bits dropped from m */
+    uint32_t q = (m + (1u << (shift - 1))) >> shift;                       /* add half, truncate: ties go outward */
+    if (e < -14) return (uint16_t)(sign | q);                              /* q may reach 0x400 = smallest normal */
+    /* q in [0x400, 0x800]; 0x800 carries into the exponent */
+    return (uint16_t)(sign | (((uint32_t)(e + 15) << 10) + (q - 0x400u)));
+}
+ORACLE_API void oracle_f32_to_f16_away(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = f32_to_f16_away(in[i]);
+}
+ORACLE_API void oracle_f32_to_bf16_away(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = f32_to_bf16_away(in[i]);
+}
+
+/* MoeGatingTopKSoftmaxV2 (moe/moe_gating_top_k_softmax_v2/README.md:12-30).
+ *   renorm 0 : p = softmax(x) (x widened to fp32, max subtracted, exp, sum, divide:
+ *              op_kernel/moe_gating_top_k_softmax_v2_ek_fullload.h:309-412); top-k of p, descending, equal values by
+ *              ascending index; softmaxOut = p when given
+ *   renorm 1 : top-k of x, then softmax over the k picked values (:414-545)
+ *   y is narrowed to x's dtype with ties away from zero (CAST_ROUND, :211-262)
+ *   finished[row] != 0 : every index of the row becomes cols (op_kernel/moe_gating_top_k_softmax_v2_perf.h:603-637)
+ * The exp/sum arithmetic and the order among equal values live in the CANN library (SoftMax, TopK, Sort32): the
+ * last-ulp behaviour here is this restatement's own. */
+ORACLE_API void oracle_moe_gating_top_k_softmax_v2(const void* x, int dtype, const uint8_t* finished, int64_t rows,
+                                                   int64_t cols, int64_t k, int64_t renorm, void* y, int32_t* idx,
+                                                   float* softmaxOut) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+        float* v = (float*)malloc(sizeof(float) * (size_t)cols);
+        char* taken = (char*)calloc((size_t)cols, 1);
+        float* picked = (float*)malloc(sizeof(float) * (size_t)k);
+        for (int64_t c = 0; c < cols; c++) v[c] = load_as_f32(x, r * cols + c, dtype);
+        if (renorm == 0) {
+            float mx = v[0];
+            double wide = 0.0;   /* the sum of the fp32 terms, rounded once: independent of any reduction order */
+            for (int64_t c = 1; c < cols; c++) mx = v[c] > mx ? v[c] : mx;
+            for (int64_t c = 0; c < cols; c++) { v[c] = expf(v[c] - mx); wide += v[c]; }
+            const float sum = (float)wide;
+            for (int64_t c = 0; c < cols; c++) { v[c] = v[c] / sum; if (softmaxOut) softmaxOut[r * cols + c] = v[c]; }
+        }
+        for (int64_t j = 0; j < k; j++) {                       /* selection: first strictly greater wins */
+            int64_t best = -1;
+            for (int64_t c = 0; c < cols; c++) {
+                if (!taken[c] && (best < 0 || v[c] > v[best])) best = c;
+            }
+            taken[best] = 1;
+            picked[j] = v[best];
+            idx[r * k + j] = (finished && finished[r]) ? (int32_t)cols : (int32_t)best;
+        }
+        if (renorm == 1) {
+            double wide = 0.0;
+            const float mx = picked[0];
+            for (int64_t j = 0; j < k; j++) { picked[j] = expf(picked[j] - mx); wide += picked[j]; }
+            const float sum = (float)wide;
+            for (int64_t j = 0; j < k; j++) picked[j] = picked[j] / sum;
+        }
+        for (int64_t j = 0; j < k; j++) {
+            if (dtype == DT_F32) ((float*)y)[r * k + j] = picked[j];
+            else if (dtype == DT_F16) ((uint16_t*)y)[r * k + j] = f32_to_f16_away(picked[j]);
+            else ((uint16_t*)y)[r * k + j] = f32_to_bf16_away(picked[j]);
+        }
+        free(v); free(taken); free(picked);
+    }
+}
+
 /* ------------------------------------------------------------------------------------------------ routing */
 
 /*

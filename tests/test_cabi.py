@@ -31,6 +31,7 @@ def test_headers_declare_the_expected_entry_points():
     names = _declared_symbols()
     for required in ["aclnnMoeInitRoutingV2GetWorkspaceSize", "aclnnMoeInitRoutingV2",
                      "aclnnMoeInitRoutingV3GetWorkspaceSize", "aclnnMoeInitRoutingV3",
+                     "aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize", "aclnnMoeGatingTopKSoftmaxV2",
                      "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize", "aclnnGroupedMatmulSwigluQuant",
                      "aclnnGroupedMatmulV4GetWorkspaceSize", "aclnnGroupedMatmulV4",
                      "aclnnGroupedMatmulV5GetWorkspaceSize", "aclnnGroupedMatmulV5",
@@ -48,7 +49,7 @@ def test_library_exports_every_declared_symbol(aclnn):
 
 
 # ------------------------------------------------------------------------------------------------ helpers
-F32, F16, I8, I32, I64, BF16 = 0, 1, 2, 3, 9, 27
+F32, F16, I8, I32, I64, BOOL, BF16 = 0, 1, 2, 3, 9, 12, 27
 
 
 class T:
@@ -124,6 +125,60 @@ def test_routing_null_and_rank_checks(aclnn):
     args[0] = x3.h
     code, msg = _status(aclnn, "aclnnMoeInitRoutingV2", args)
     assert code == INVALID and "dim number of x should be 2" in msg
+
+
+# ------------------------------------------------------------------------------------------------ gating
+def _gating_args(aclnn, shape=(6, 16), k=4, renorm=0, flag=False, dtype=F32, finished=False, **over):
+    x = T(aclnn, shape, dtype)
+    fin = T(aclnn, over.get("fin_shape", shape[:-1]), over.get("fin_dtype", BOOL)) if finished else None
+    y = T(aclnn, over.get("y_shape", tuple(shape[:-1]) + (k,)), over.get("y_dtype", dtype))
+    idx = T(aclnn, over.get("idx_shape", tuple(shape[:-1]) + (k,)), over.get("idx_dtype", I32))
+    sm = T(aclnn, over.get("sm_shape", shape), over.get("sm_dtype", F32)) if over.get("with_sm", flag) else None
+    return [x.h, fin.h if fin else None, k, renorm, flag, y.h, idx.h, sm.h if sm else None]
+
+
+def test_gating_valid(aclnn):
+    for kw in [dict(), dict(renorm=1), dict(flag=True), dict(renorm=1, flag=True, with_sm=False), dict(dtype=F16),
+               dict(dtype=BF16, finished=True), dict(shape=(2, 3, 16)), dict(shape=(2, 3, 16), finished=True, flag=True),
+               dict(shape=(0, 16)), dict(k=16), dict(shape=(4, 32768), k=1024)]:
+        code, ws = _status(aclnn, "aclnnMoeGatingTopKSoftmaxV2", _gating_args(aclnn, **kw))
+        assert code == 0 and ws == 0, (kw, ws)
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    # rules and messages of moe/moe_gating_top_k_softmax_v2/op_host/moe_gating_top_k_softmax_v2_tiling_base.cpp:40-260
+    (dict(dtype=I8), "only supports float32,half,bf16"),
+    (dict(shape=(16,), y_shape=(4,), idx_shape=(4,)), "x shape dim(=1) is not 2 or 3"),
+    (dict(shape=(2, 2, 2, 16)), "x shape dim(=4) is not 2 or 3"),
+    (dict(shape=(6, 0), k=1), "last dim is zero"),
+    (dict(finished=True, fin_dtype=I8), "should be BOOL"),
+    (dict(finished=True, fin_shape=(6, 1)), "finished dim num (=2) error, should be (=1)"),
+    (dict(finished=True, fin_shape=(5,)), "finished and x shape not equal"),
+    (dict(k=0), "attr k(=0) is wrong"),
+    (dict(k=17), "attr k(=17) is wrong"),
+    (dict(shape=(2, 4096), k=1025), "attr k(=1025) is too large"),
+    (dict(renorm=2), "attr renorm(=2) is wrong"),
+    (dict(y_dtype=F16), "should be same with x data type"),
+    (dict(y_shape=(6, 5)), "with last dim k"),
+    (dict(y_shape=(5, 4)), "with last dim k"),
+    (dict(idx_dtype=I64), "only supports int32"),
+    (dict(idx_shape=(6, 3)), "with last dim k"),
+    (dict(flag=True, sm_dtype=F16), "should be float"),
+    (dict(flag=True, sm_shape=(6, 15)), "softmaxResult and x shape not equal"),
+    (dict(shape=(2, 32769)), "at most 32768 experts"),
+])
+def test_gating_invalid(aclnn, kw, fragment):
+    code, msg = _status(aclnn, "aclnnMoeGatingTopKSoftmaxV2", _gating_args(aclnn, **kw))
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_gating_nulls(aclnn):
+    for pos in (0, 5, 6):
+        args = _gating_args(aclnn)
+        args[pos] = None
+        assert _status(aclnn, "aclnnMoeGatingTopKSoftmaxV2", args)[0] == NULLPTR, pos
+    args = _gating_args(aclnn, flag=True, with_sm=False)       # softmax output requested, no tensor for it
+    assert _status(aclnn, "aclnnMoeGatingTopKSoftmaxV2", args)[0] == NULLPTR
 
 
 # ------------------------------------------------------------------------------------------------ routing V3
@@ -317,7 +372,7 @@ def test_gmm_v5_takes_a_tuning_hint(aclnn):
 
 
 def test_reference_examples_compile_and_link_unmodified():
-    """The four example programs of the reference for the operators on the path build against include/ and link to
+    """The reference's example programs for the operators built here build against include/ and link to
     libcust_opapi.so without a change (needs the reference checkout; the binaries are run by the GPU tests)."""
     import subprocess
     if not os.path.isdir("/root/reference/moe/moe_init_routing_v2/examples"):
@@ -326,7 +381,8 @@ def test_reference_examples_compile_and_link_unmodified():
                          stderr=subprocess.STDOUT, text=True)
     assert res.returncode == 0, res.stdout
     for name in ("test_aclnn_moe_init_routing_v2", "test_aclnn_grouped_matmul_swiglu_quant", "test_aclnn_grouped_matmul",
-                 "test_aclnn_moe_finalize_routing_v2"):
+                 "test_aclnn_moe_finalize_routing_v2", "test_aclnn_moe_init_routing_v3",
+                 "test_aclnn_moe_gating_top_k_softmax_v2"):
         assert os.access(os.path.join(ROOT, "oracle", "_ref", "examples", name), os.X_OK), name
 
 

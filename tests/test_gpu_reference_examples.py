@@ -3,11 +3,13 @@ libcust_opapi.so (recipe: `make -C oracle ref_examples`, binaries in oracle/_ref
 
   moe/moe_init_routing_v2/examples/test_aclnn_moe_init_routing_v2.cpp        drop/pad routing of 3 tokens, E=3, C=2
   moe/moe_finalize_routing_v2/examples/test_aclnn_moe_finalize_routing_v2.cpp fp32 finalize with x1, x2, bias
+  moe/moe_gating_top_k_softmax_v2/examples/test_aclnn_moe_gating_top_k_softmax_v2.cpp   softmax then top-2 of 3x4 logits
   gmm/grouped_matmul/examples/test_aclnn_grouped_matmul.cpp                   fp16 grouped matmul via V5
   gmm/grouped_matmul_swiglu_quant/examples/test_aclnn_grouped_matmul_swiglu_quant.cpp   FRACTAL_NZ weight
+  moe/moe_init_routing_v3/examples/test_aclnn_moe_init_routing_v3.cpp         FLOAT rows into an INT8 output, quantMode -1
 
-The first two must print what the oracle computes from the same literals (held below as data).  The last two use a
-data type / weight format outside this build's path: they must fail cleanly in the first phase with
+The first three must print what the oracle computes from the same literals (held below as data).  The last three use a
+data type / weight format / dtype pairing outside this build's path: they must fail cleanly in the first phase with
 ACLNN_ERR_PARAM_INVALID (161002), the reference's code for an unsupported combination, not crash.
 """
 import os
@@ -64,7 +66,18 @@ def test_finalize_example(oracle, dev):
     np.testing.assert_allclose(got, want.reshape(-1), rtol=0, atol=5e-6)  # six printed decimals of values up to ~50
 
 
+def test_gating_example(oracle, dev):
+    rc, text = _run("test_aclnn_moe_gating_top_k_softmax_v2")
+    assert rc == 0, text
+    x = np.array([0.1, 1.1, 2.1, 3.1, 4.1, 5.1, 6.1, 7.1, 8.1, 9.1, 10.1, 11.1], np.float32).reshape(3, 4)
+    want, _, _ = oracle.moe_gating_top_k_softmax_v2(x, 2, 0)
+    got = np.array(_values(text, "result", float), np.float32)
+    assert got.shape == (6,)
+    np.testing.assert_allclose(got, want.reshape(-1), rtol=0, atol=1e-6)   # six printed decimals
+
+
 @pytest.mark.parametrize("name,api", [("test_aclnn_grouped_matmul", "aclnnGroupedMatmulV5GetWorkspaceSize"),
+                                      ("test_aclnn_moe_init_routing_v3", "aclnnMoeInitRoutingV3GetWorkspaceSize"),
                                       ("test_aclnn_grouped_matmul_swiglu_quant",
                                        "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize")])
 def test_unsupported_examples_fail_cleanly(name, api, dev):
