@@ -10,10 +10,16 @@
  * key/value pairs (type 2, op_kernel/moe_v3_expert_tokens_count.h:254-269), and the index output is either the
  * scatter-type map of V2 (rowIdxType 1: [source] -> destination) or the gather-type map (0: [destination] -> source).
  *
- * This build: quantMode -1 only (dynamic quantisation, quantMode 1, is rejected with ACLNN_ERR_PARAM_INVALID);
- * at most 2047 active experts when the range is a proper sub-range, 2048 otherwise; expertTokensNumType 0 (cumsum) is
- * accepted as an extension (the reference's tiling rejects it although the operator definition lists it), because
- * aclnnGroupedMatmulSwigluQuant takes a cumsum group list.
+ * quantMode 1 (dynamic quantisation, op_kernel/moe_v3_gather_dynamic_quant.h:103-141): x is FLOAT/FLOAT16/BF16,
+ * scaleOptional is the optional smooth scale [end - start, H] multiplied into the row of the expert it is routed to,
+ * expandedXOut is INT8 with per-row scale max|v| / 127 in expandedScaleOut (always written): v / scale by true division,
+ * narrowed to half precision toward zero, then to INT8 with halves away from zero.  A row of zeros gives scale 0 and
+ * zeros (the reference divides 0 by 0 there).
+ *
+ * This build: at most 2047 active experts when the range is a proper sub-range, 2048 otherwise; expertTokensNumType 0
+ * (cumsum) is accepted as an extension (the reference's tiling rejects it although the operator definition lists it),
+ * because aclnnGroupedMatmulSwigluQuant takes a cumsum group list; offsetOptional is accepted and ignored, as in the
+ * reference.
  */
 #ifndef OPS_TRANSFORMER_AMD_ACLNN_MOE_INIT_ROUTING_V3_H_
 #define OPS_TRANSFORMER_AMD_ACLNN_MOE_INIT_ROUTING_V3_H_

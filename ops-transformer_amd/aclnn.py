@@ -281,7 +281,9 @@ def moe_gating_top_k_softmax_v2(x, k, renorm=0, finished=None, output_softmax=Fa
 
 def moe_init_routing_v3(x, expert_idx, scale=None, expert_num=0, expert_tokens_num_type=1, quant_mode=-1,
                         active_expert_range=None, row_idx_type=1, active_num=-1, out=None, workspace=None):
-    """aclnnMoeInitRoutingV3 (dropless).  Returns (expandedX, expandedRowIdx, tokenCounts int64, expandedScale or None)."""
+    """aclnnMoeInitRoutingV3 (dropless).  Returns (expandedX, expandedRowIdx, tokenCounts int64, expandedScale or None).
+    quant_mode -1: scale is the optional per-token scale [T]; quant_mode 1 (dynamic quantisation to int8): scale is the
+    optional smooth scale [active experts, H] and expandedScale is always produced."""
     T, H = x.shape
     K = expert_idx.shape[1]
     dev = x.device
@@ -289,10 +291,11 @@ def moe_init_routing_v3(x, expert_idx, scale=None, expert_num=0, expert_tokens_n
     if out is not None:
         expanded_x, row_idx, counts, expanded_scale = out
     else:
-        expanded_x = torch.zeros((T * K, H), dtype=x.dtype, device=dev)
+        expanded_x = torch.zeros((T * K, H), dtype=torch.int8 if quant_mode == 1 else x.dtype, device=dev)
         row_idx = torch.empty((T * K,), dtype=torch.int32, device=dev)
         counts = torch.zeros((expert_num, 2) if expert_tokens_num_type == 2 else (end - start,), dtype=torch.int64, device=dev)
-        expanded_scale = None if scale is None else torch.zeros((T * K,), dtype=torch.float32, device=dev)
+        expanded_scale = (torch.zeros((T * K,), dtype=torch.float32, device=dev)
+                          if (scale is not None or quant_mode == 1) else None)
     h = _Handles()
     try:
         args = [h.tensor(x), h.tensor(expert_idx), h.tensor(scale), None, active_num, 0, expert_num, 0,

@@ -22,6 +22,8 @@
 // The gather reads each source row once with 16-byte lanes and writes its K destinations.
 #include "opapi_common.h"
 
+#include <hip/hip_fp16.h>
+
 #include "aclnnop/aclnn_moe_init_routing_v2.h"
 #include "aclnnop/aclnn_moe_init_routing_v3.h"
 
@@ -357,6 +359,120 @@ __global__ __launch_bounds__(1024) void CountV3Kernel(CountV3Args a) {
     }
 }
 
+// V3 dynamic quantisation (quantMode 1), fused with the row gather.  Per destination row:
+//   v = float(x[token, :]) * smooth[expert - start, :] (smooth optional);  s = max|v| / 127;  expandedScale[dst] = s;
+//   expandedX[dst, :] = int8(round_half_away(fp16_toward_zero(v / s)))      (true divide)
+// as moe/moe_init_routing_v3/op_kernel/moe_v3_gather_dynamic_quant.h:103-141 does.  A row of zeros gives s = 0 and
+// zeros (the reference divides 0 by 0 there).  One workgroup per token; without a smooth scale the K copies of a token
+// are identical, so the row is quantised once and written K times.  The row is read twice (maximum, then quantise):
+// the second read comes from cache.
+struct QuantGatherArgs {
+    const void* x;
+    int8_t* expandedX;
+    float* expandedScale;
+    const int32_t* expandedRowIdx;  // scatter-type map
+    const int32_t* expertIdx;
+    const float* smooth;            // [active, cols] or nullptr
+    int64_t cols;
+    int32_t topK;
+    int32_t expertStart;
+    int32_t dtype;                  // ACL_FLOAT, ACL_FLOAT16, ACL_BF16
+};
+
+__device__ __forceinline__ float LoadAsFloat(const void* p, int64_t i, int dtype) {
+    if (dtype == ACL_FLOAT) return static_cast<const float*>(p)[i];
+    const uint16_t raw = static_cast<const uint16_t*>(p)[i];
+    if (dtype == ACL_FLOAT16) return __half2float(__ushort_as_half(raw));
+    return __uint_as_float(static_cast<uint32_t>(raw) << 16);
+}
+
+// kVec consecutive elements starting at element i (kVec 4: i is a multiple of 4 and the buffer is 16-byte aligned).
+template <int kVec>
+__device__ __forceinline__ void LoadRowChunk(const void* p, int64_t i, int dtype, float (&v)[kVec]) {
+    if constexpr (kVec == 4) {
+        if (dtype == ACL_FLOAT) {
+            const float4 f = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i);
+            v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+        } else {
+            const uint2 u = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(p) + i);
+            const uint16_t raw[4] = {static_cast<uint16_t>(u.x), static_cast<uint16_t>(u.x >> 16),
+                                     static_cast<uint16_t>(u.y), static_cast<uint16_t>(u.y >> 16)};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] = dtype == ACL_FLOAT16 ? __half2float(__ushort_as_half(raw[e]))
+                                            : __uint_as_float(static_cast<uint32_t>(raw[e]) << 16);
+            }
+        }
+    } else {
+        v[0] = LoadAsFloat(p, i, dtype);
+    }
+}
+
+__device__ __forceinline__ int8_t QuantizeOne(float v, float scale) {
+    const float h = __half2float(__float2half_rz(v / scale));
+    float r = truncf(h + copysignf(0.5f, h));
+    r = fminf(fmaxf(r, -128.f), 127.f);
+    return static_cast<int8_t>(static_cast<int>(r));
+}
+
+template <int kVec>
+__global__ __launch_bounds__(kGatherThreads) void QuantGatherRowsKernel(QuantGatherArgs a) {
+    __shared__ float waveMax[kGatherThreads / kWaveSize];
+    const int64_t n = blockIdx.x;
+    const int copies = a.smooth != nullptr ? a.topK : 1;
+    for (int j = 0; j < copies; ++j) {
+        const int32_t dstOne = a.expandedRowIdx[n * a.topK + j];
+        if (a.smooth != nullptr && dstOne < 0) continue;  // uniform over the workgroup
+        const float* smooth =
+            a.smooth != nullptr ? a.smooth + static_cast<int64_t>(a.expertIdx[n * a.topK + j] - a.expertStart) * a.cols : nullptr;
+        float mx = 0.f;
+        for (int64_t c = static_cast<int64_t>(threadIdx.x) * kVec; c < a.cols; c += kGatherThreads * kVec) {
+            float v[kVec];
+            LoadRowChunk<kVec>(a.x, n * a.cols + c, a.dtype, v);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                if (smooth != nullptr) v[i] = v[i] * smooth[c + i];
+                mx = fmaxf(mx, fabsf(v[i]));
+            }
+        }
+        for (int d = 32; d > 0; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+        __syncthreads();  // the previous copy's readers of waveMax are done
+        if (threadIdx.x % kWaveSize == 0) waveMax[threadIdx.x / kWaveSize] = mx;
+        __syncthreads();
+        mx = waveMax[0];
+        for (int w = 1; w < kGatherThreads / kWaveSize; ++w) mx = fmaxf(mx, waveMax[w]);
+        const float scale = mx / 127.0f;
+
+        for (int jj = (a.smooth != nullptr ? j : 0); jj < (a.smooth != nullptr ? j + 1 : a.topK); ++jj) {
+            const int32_t dst = a.expandedRowIdx[n * a.topK + jj];
+            if (dst >= 0 && threadIdx.x == 0) a.expandedScale[dst] = scale;
+        }
+        for (int64_t c = static_cast<int64_t>(threadIdx.x) * kVec; c < a.cols; c += kGatherThreads * kVec) {
+            int8_t q[kVec];
+            float v[kVec];
+            LoadRowChunk<kVec>(a.x, n * a.cols + c, a.dtype, v);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                if (smooth != nullptr) v[i] = v[i] * smooth[c + i];
+                q[i] = mx == 0.f ? static_cast<int8_t>(0) : QuantizeOne(v[i], scale);
+            }
+            for (int jj = (a.smooth != nullptr ? j : 0); jj < (a.smooth != nullptr ? j + 1 : a.topK); ++jj) {
+                const int64_t dst = a.expandedRowIdx[n * a.topK + jj];
+                if (dst < 0) continue;
+                int8_t* out = a.expandedX + dst * a.cols + c;
+                if constexpr (kVec == 4) {
+                    *reinterpret_cast<uint32_t*>(out) = static_cast<uint32_t>(static_cast<uint8_t>(q[0])) |
+                                                        (static_cast<uint32_t>(static_cast<uint8_t>(q[1])) << 8) |
+                                                        (static_cast<uint32_t>(static_cast<uint8_t>(q[2])) << 16) |
+                                                        (static_cast<uint32_t>(static_cast<uint8_t>(q[3])) << 24);
+                } else {
+                    out[0] = q[0];
+                }
+            }
+        }
+    }
+}
+
 // V3: expandedScale[destination] = scale[source / K] through the scatter-type map.
 __global__ void ScatterScaleKernel(const float* scale, float* expandedScale, const int32_t* rowIdx, int64_t total,
                                    int32_t topK) {
@@ -394,6 +510,9 @@ class InitRoutingExecutor : public aclOpExecutor {
     int32_t kvPairs = 0;
     const float* scale = nullptr;
     float* expandedScale = nullptr;
+    bool dynamicQuant = false;                // quantMode 1: `scale` is the optional smooth scale [active, cols]
+    int32_t xDtype = ACL_FLOAT;
+    int64_t cols = 0;
     uint64_t offRemapKeys = 0, offCounts = 0, offScatterMap = 0;
     // plan
     int passes = 1;
@@ -533,10 +652,22 @@ class InitRoutingExecutor : public aclOpExecutor {
         if (v3) {
             CountV3Args ca{countOrCumsum, count64, expertEnd - expertStart, expertStart, countMode, kvPairs};
             hipLaunchKernelGGL(CountV3Kernel, dim3(1), dim3(1024), 0, stream, ca);
-            if (scale != nullptr && !(rowBytes > 0 && tokens > 0)) {  // otherwise the row gather carries the scales
+            if (scale != nullptr && !dynamicQuant && !(rowBytes > 0 && tokens > 0)) {  // otherwise the row gather carries the scales
                 hipLaunchKernelGGL(ScatterScaleKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
                                    stream, scale, expandedScale, expandedRowIdx, total, static_cast<int32_t>(topK));
             }
+        }
+        if (dynamicQuant) {
+            if (tokens > 0 && cols > 0) {
+                opapi::KernelTimer timer("routing_quant_gather", stream);
+                QuantGatherArgs q{x, reinterpret_cast<int8_t*>(expandedX), expandedScale, expandedRowIdx, expertIdx, scale,
+                                  cols, static_cast<int32_t>(topK), expertStart, xDtype};
+                const bool wide = cols % 4 == 0 && reinterpret_cast<uintptr_t>(expandedX) % 4 == 0 &&
+                                  reinterpret_cast<uintptr_t>(x) % 16 == 0;
+                if (wide) hipLaunchKernelGGL(QuantGatherRowsKernel<4>, dim3(static_cast<unsigned>(tokens)), dim3(kGatherThreads), 0, stream, q);
+                else hipLaunchKernelGGL(QuantGatherRowsKernel<1>, dim3(static_cast<unsigned>(tokens)), dim3(kGatherThreads), 0, stream, q);
+            }
+            return ACLNN_SUCCESS;
         }
         if (rowBytes > 0 && tokens > 0) {
             opapi::KernelTimer timer("routing_gather", stream);
@@ -708,13 +839,14 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
                 "expert_end should be less than or equal to %d%s", expertTokensNumType == 2 ? 5120 : 10240,
                 expertTokensNumType == 2 ? " in KEY_VALUE mode" : "");
     OPAPI_CHECK(quantMode == -1 || quantMode == 1, kInvalid, "quant_mode currently support -1 or 1");
-    OPAPI_CHECK(quantMode == -1, kInvalid, "quant_mode 1 (dynamic quantisation) is not supported in this build");
+    const bool dynamicQuant = quantMode == 1;
     OPAPI_CHECK(rowIdxType == 0 || rowIdxType == 1, kInvalid, "row_idx_type currently support 1 or 0");
     // offset only matters to static quantisation; like the reference, accept a FLOAT tensor and ignore it
     OPAPI_CHECK(offsetOptional == nullptr || offsetOptional->dtype == ACL_FLOAT, kInvalid, "offset must be FLOAT");
 
     OPAPI_CHECK(x->dtype == ACL_FLOAT || x->dtype == ACL_FLOAT16 || x->dtype == ACL_BF16 || x->dtype == ACL_INT8, kInvalid,
                 "x dtype %d is not supported (FLOAT, FLOAT16, BF16, INT8)", (int)x->dtype);
+    OPAPI_CHECK(!(dynamicQuant && x->dtype == ACL_INT8), kInvalid, "quant_mode 1 quantises FLOAT, FLOAT16 or BF16 rows, not INT8");
     OPAPI_CHECK(expertIdx->dtype == ACL_INT32, kInvalid, "expertIdx must be INT32");
     OPAPI_CHECK(x->dims.size() == 2, kInvalid, "The dim number of x should be 2.");
     OPAPI_CHECK(expertIdx->dims.size() == 2, kInvalid, "The dim number of expert_idx should be 2.");
@@ -730,16 +862,27 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
                 "this build routes at most %d active experts (%d when the range is a proper sub-range)", kMaxBins,
                 kMaxBins - 1);
 
-    if (scaleOptional != nullptr) {
+    if (dynamicQuant && scaleOptional != nullptr) {  // smooth scale, one row per active expert
+        OPAPI_CHECK(scaleOptional->dtype == ACL_FLOAT, kInvalid, "scale must be FLOAT");
+        OPAPI_CHECK(scaleOptional->dims.size() == 2, kInvalid, "The dim number of scale should be 2.");
+        OPAPI_CHECK(scaleOptional->dims[0] == active, kInvalid, "The first dim of scale should be %lld", (long long)active);
+        OPAPI_CHECK(scaleOptional->dims[1] == cols, kInvalid, "The second dim of scale should be %lld", (long long)cols);
+    }
+    if (!dynamicQuant && scaleOptional != nullptr) {
         OPAPI_CHECK(scaleOptional->dtype == ACL_FLOAT, kInvalid, "scale must be FLOAT");
         OPAPI_CHECK(scaleOptional->dims.size() == 1, kInvalid, "The dim number of scale should be 1.");
         OPAPI_CHECK(scaleOptional->dims[0] == tokens, kInvalid, "The first dim of scale should be %lld", (long long)tokens);
-        OPAPI_CHECK(expandedScaleOut != nullptr, ACLNN_ERR_PARAM_NULLPTR, "expandedScaleOut must not be null when scale is given");
+    }
+    if (dynamicQuant || scaleOptional != nullptr) {
+        OPAPI_CHECK(expandedScaleOut != nullptr, ACLNN_ERR_PARAM_NULLPTR,
+                    "expandedScaleOut must not be null when scale is given or quant_mode is 1");
         OPAPI_CHECK(expandedScaleOut->dtype == ACL_FLOAT && expandedScaleOut->dims.size() == 1 &&
                         expandedScaleOut->dims[0] == total, kInvalid, "expandedScaleOut must be FLOAT [%lld]", (long long)total);
-        OPAPI_CHECK(IsContiguous(scaleOptional) && IsContiguous(expandedScaleOut), kInvalid, "scale tensors must be contiguous");
+        OPAPI_CHECK((scaleOptional == nullptr || IsContiguous(scaleOptional)) && IsContiguous(expandedScaleOut), kInvalid,
+                    "scale tensors must be contiguous");
     }
-    OPAPI_CHECK(expandedXOut->dtype == x->dtype, kInvalid, "expandedXOut dtype must equal x dtype without quantisation");
+    if (dynamicQuant) OPAPI_CHECK(expandedXOut->dtype == ACL_INT8, kInvalid, "expandedXOut must be INT8 when quant_mode is 1");
+    else OPAPI_CHECK(expandedXOut->dtype == x->dtype, kInvalid, "expandedXOut dtype must equal x dtype without quantisation");
     OPAPI_CHECK(expandedXOut->dims.size() == 2 && expandedXOut->dims[0] == total && expandedXOut->dims[1] == cols, kInvalid,
                 "expandedXOut must be [%lld, %lld]", (long long)total, (long long)cols);
     OPAPI_CHECK(expandedRowIdxOut->dtype == ACL_INT32 && expandedRowIdxOut->dims.size() == 1 &&
@@ -762,8 +905,10 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
                     "expertIdx / expandedRowIdxOut carry no device memory");
         OPAPI_CHECK(cols == 0 || (x->data != nullptr && expandedXOut->data != nullptr), ACLNN_ERR_PARAM_NULLPTR,
                     "x / expandedXOut carry no device memory");
-        OPAPI_CHECK(scaleOptional == nullptr || (scaleOptional->data != nullptr && expandedScaleOut->data != nullptr),
-                    ACLNN_ERR_PARAM_NULLPTR, "scale / expandedScaleOut carry no device memory");
+        OPAPI_CHECK(scaleOptional == nullptr || scaleOptional->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
+                    "scale carries no device memory");
+        OPAPI_CHECK(!(dynamicQuant || scaleOptional != nullptr) || expandedScaleOut->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
+                    "expandedScaleOut carries no device memory");
     }
 
     auto* ex = new (std::nothrow) InitRoutingExecutor();
@@ -779,7 +924,10 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
     // key/value pairs written: min(active + 1, expertNum), as the reference sizes its copy-out
     ex->kvPairs = static_cast<int32_t>(active + 1 < expertNum ? active + 1 : expertNum);
     ex->scale = scaleOptional != nullptr ? reinterpret_cast<const float*>(DataPtr(scaleOptional)) : nullptr;
-    ex->expandedScale = scaleOptional != nullptr ? reinterpret_cast<float*>(DataPtr(expandedScaleOut)) : nullptr;
+    ex->expandedScale = (dynamicQuant || scaleOptional != nullptr) ? reinterpret_cast<float*>(DataPtr(expandedScaleOut)) : nullptr;
+    ex->dynamicQuant = dynamicQuant;
+    ex->xDtype = x->dtype;
+    ex->cols = cols;
     ex->expertStart = static_cast<int32_t>(expertStart);
     ex->expertEnd = static_cast<int32_t>(expertEnd);
     ex->remap = remap;

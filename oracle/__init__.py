@@ -183,6 +183,35 @@ def moe_init_routing_v3(x, expert_idx, scale=None, expert_num=0, expert_range=No
     return ex, out_idx, counts, ex_scale
 
 
+def f32_to_f16_trunc_value(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, np.float32)
+    lib().oracle_f32_to_f16_trunc_value(_p(a), _p(out), ctypes.c_int64(a.size))
+    return out
+
+
+def moe_init_routing_v3_quant(x, expert_idx, smooth=None, expert_num=0, expert_range=None, count_mode=1, row_idx_type=1,
+                              dtype=DT_F32):
+    """MoeInitRoutingV3 with quantMode 1.  x: fp32, or uint16 bit patterns for DT_F16 / DT_BF16.
+    Returns (expandedX int8 [M, cols], idx int32 [M], counts int64, expandedScale fp32 [M]); unrouted rows are zero."""
+    x = _c(x)
+    T, cols = x.shape
+    idx = _c(expert_idx, np.int32)
+    K = idx.shape[1]
+    M = T * K
+    start, end = (0, expert_num) if expert_range is None else expert_range
+    ex = np.zeros((M, cols), np.int8)
+    out_idx = np.zeros((M,), np.int32)
+    counts = np.zeros((expert_num, 2) if count_mode == 2 else (end - start,), np.int64)
+    ex_scale = np.zeros((M,), np.float32)
+    sm = None if smooth is None else _c(smooth, np.float32)
+    lib().oracle_moe_init_routing_v3_quant(
+        _p(x), ctypes.c_int(dtype), ctypes.c_int64(cols), _p(idx), _p(sm), ctypes.c_int64(T), ctypes.c_int64(K),
+        ctypes.c_int64(expert_num), ctypes.c_int64(start), ctypes.c_int64(end), ctypes.c_int64(count_mode),
+        ctypes.c_int64(row_idx_type), _p(ex), _p(out_idx), _p(counts), _p(ex_scale))
+    return ex, out_idx, counts, ex_scale
+
+
 # ----------------------------------------------------------------------------------------------- GEMMs
 def _gemm_common(x, w, w_trans, group_list, rows):
     x = _c(x, np.int8)

@@ -310,6 +310,65 @@ ORACLE_API int oracle_moe_init_routing_v3(const void* x, int64_t rowBytes, const
     return 0;
 }
 
+/* fp32 -> fp16 toward zero (Ascend C CAST_TRUNC), on the magnitude bits; the result decoded back to fp32. */
+static inline float f32_to_f16_trunc_value(float f) {
+    const uint32_t u = f2u(f), sign = u & 0x80000000u, mag = u & 0x7fffffffu;
+    if (mag >= 0x7f800000u) return f;                                      /* inf / nan pass through */
+    if (mag >= 0x477fe000u) return u2f(sign | 0x477fe000u);                /* beyond 65504: clamp to the largest half */
+    const int32_t e = (int32_t)(mag >> 23) - 127;
+    if (e < -24) return u2f(sign);                                          /* below the smallest subnormal */
+    const int drop = e < -14 ? 13 + (-14 - e) : 13;                         /* mantissa bits a half cannot hold */
+    const uint32_t m = (mag & 0x7fffffu) | 0x800000u;
+    const uint32_t kept = (m >> drop) << drop;                              /* chop */
+    if (kept == 0) return u2f(sign);
+    /* rebuild: value = kept * 2^(e-23) */
+    return u2f(sign | f2u(ldexpf((float)kept, e - 23)));
+}
+
+/* MoeInitRoutingV3 with dynamic quantisation (quantMode 1): routing as oracle_moe_init_routing_v3, and per routed row
+ *   v = float(x[token,:]) * smooth[expert - start,:] (smooth optional);  s = max|v| / 127;  q = v / s (true divide);
+ *   expandedX[dst,:] = int8(round-half-away(fp16-toward-zero(q)));  expandedScale[dst] = s
+ * (moe/moe_init_routing_v3/op_kernel/moe_v3_gather_dynamic_quant.h:103-141).  A row of zeros: s = 0, zeros (the
+ * reference computes 0/0 there). */
+ORACLE_API int oracle_moe_init_routing_v3_quant(const void* x, int dtype, int64_t cols, const int32_t* expertIdx,
+                                                const float* smooth, int64_t T, int64_t K, int64_t expertNum, int64_t start,
+                                                int64_t end, int64_t countMode, int64_t rowIdxType, int8_t* expandedX,
+                                                int32_t* idxOut, int64_t* counts, float* expandedScale) {
+    const int64_t M = T * K;
+    int32_t* scatter = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M > 0 ? M : 1));
+    oracle_moe_init_routing_v3(NULL, 0, expertIdx, NULL, T, K, expertNum, start, end, countMode, 1, NULL, scatter, counts, NULL);
+    if (rowIdxType == 0) for (int64_t i = 0; i < M; i++) idxOut[i] = -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; i++) {
+        const int64_t d = scatter[i];
+        if (rowIdxType == 1) idxOut[i] = (int32_t)d;
+        if (d < 0) continue;
+        if (rowIdxType == 0) idxOut[d] = (int32_t)i;
+        const float* sm = smooth ? smooth + (expertIdx[i] - start) * cols : NULL;
+        float mx = 0.f;
+        for (int64_t c = 0; c < cols; c++) {
+            float v = load_as_f32(x, (i / K) * cols + c, dtype);
+            if (sm) v = v * sm[c];
+            mx = fabsf(v) > mx ? fabsf(v) : mx;
+        }
+        const float s = mx / 127.0f;
+        expandedScale[d] = s;
+        for (int64_t c = 0; c < cols; c++) {
+            float v = load_as_f32(x, (i / K) * cols + c, dtype);
+            if (sm) v = v * sm[c];
+            float r = mx == 0.f ? 0.f : roundf(f32_to_f16_trunc_value(v / s));   /* roundf: halves away from zero */
+            r = r > 127.f ? 127.f : (r < -128.f ? -128.f : r);
+            expandedX[d * cols + c] = (int8_t)r;
+        }
+    }
+    free(scatter);
+    return 0;
+}
+
+ORACLE_API void oracle_f32_to_f16_trunc_value(const float* in, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = f32_to_f16_trunc_value(in[i]);
+}
+
 /* ------------------------------------------------------------------------------------------------ grouped GEMM */
 
 /* Group boundaries from groupList: type 0 = inclusive cumsum, type 1 = per-group counts (grouped_matmul_utils.h:243-257). */

@@ -191,7 +191,7 @@ def _routing_v3_args(aclnn, T_=8, K=2, H=16, E=4, rng=None, num_type=1, flag=Tru
     ex = T(aclnn, over.get("ex_shape", (T_ * K, H)), over.get("ex_dtype", x_dtype))
     ri = T(aclnn, over.get("ri_shape", (T_ * K,)), I32)
     cnt = T(aclnn, over.get("cnt_shape", (E, 2) if num_type == 2 else (max(end - start, 0),)), over.get("cnt_dtype", I64))
-    es = T(aclnn, (T_ * K,), F32) if with_scale else None
+    es = T(aclnn, (T_ * K,), F32) if (with_scale or over.get("with_es")) else None
     arr = None if rng is None else aclnn.lib().aclCreateIntArray((ctypes.c_int64 * len(rng))(*rng), len(rng))
     return [x.h, idx.h, scale.h if scale else None, None, active, 0, E, mode, num_type, flag, quant, arr, row_idx_type,
             ex.h, ri.h, cnt.h, es.h if es else None]
@@ -199,7 +199,10 @@ def _routing_v3_args(aclnn, T_=8, K=2, H=16, E=4, rng=None, num_type=1, flag=Tru
 
 def test_routing_v3_valid(aclnn):
     for kw in [dict(), dict(num_type=0), dict(num_type=2), dict(rng=(1, 3)), dict(row_idx_type=0), dict(active=16),
-               dict(x_dtype=BF16, with_scale=False), dict(T_=0), dict(E=2048), dict(E=4096, rng=(100, 2147))]:
+               dict(x_dtype=BF16, with_scale=False), dict(T_=0), dict(E=2048), dict(E=4096, rng=(100, 2147)),
+               dict(quant=1, x_dtype=BF16, ex_dtype=I8, scale_shape=(4, 16)),
+               dict(quant=1, x_dtype=F32, ex_dtype=I8, rng=(1, 3), scale_shape=(2, 16)),
+               dict(quant=1, x_dtype=F16, ex_dtype=I8, with_scale=False, with_es=True)]:
         code, ws = _status(aclnn, "aclnnMoeInitRoutingV3", _routing_v3_args(aclnn, **kw))
         assert code == 0, (kw, ws)
 
@@ -217,7 +220,11 @@ def test_routing_v3_valid(aclnn):
     (dict(rng=(0, 5)), "expert_end should be less than or equal to 4"),
     (dict(rng=(0, 1, 2)), "dim number of expert_range should be 2"),
     (dict(quant=0), "quant_mode currently support -1 or 1"),
-    (dict(quant=1), "not supported in this build"),
+    (dict(quant=1), "not INT8"),                                   # dynamic quantisation needs float rows
+    (dict(quant=1, x_dtype=BF16, ex_dtype=BF16, scale_shape=(4, 16)), "expandedXOut must be INT8"),
+    (dict(quant=1, x_dtype=BF16, ex_dtype=I8, scale_shape=(8,)), "dim number of scale should be 2"),
+    (dict(quant=1, x_dtype=BF16, ex_dtype=I8, scale_shape=(3, 16)), "first dim of scale should be 4"),
+    (dict(quant=1, x_dtype=BF16, ex_dtype=I8, scale_shape=(4, 15)), "second dim of scale should be 16"),
     (dict(row_idx_type=2), "row_idx_type currently support 1 or 0"),
     (dict(scale_shape=(9,)), "first dim of scale should be 8"),
     (dict(scale_shape=(8, 1)), "dim number of scale should be 1"),
@@ -241,6 +248,8 @@ def test_routing_v3_nulls(aclnn):
         assert _status(aclnn, "aclnnMoeInitRoutingV3", args)[0] == NULLPTR, pos
     args = _routing_v3_args(aclnn)
     args[16] = None                      # scale given, no place for the routed scales
+    assert _status(aclnn, "aclnnMoeInitRoutingV3", args)[0] == NULLPTR
+    args = _routing_v3_args(aclnn, quant=1, x_dtype=BF16, ex_dtype=I8, with_scale=False)   # quantisation always emits scales
     assert _status(aclnn, "aclnnMoeInitRoutingV3", args)[0] == NULLPTR
 
 

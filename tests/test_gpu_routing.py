@@ -188,3 +188,59 @@ def test_v3_skewed_routing_matches_v2(pkg, aclnn, dev):
     ex3, ri3, cum3, _ = _run_v3(aclnn, dev, x, idx, None, expert_num=cfg.experts, expert_tokens_num_type=0)
     assert np.array_equal(ri2, ri3) and np.array_equal(cum2.astype(np.int64), cum3)
     assert np.array_equal(ex2.view(np.uint32), ex3.view(np.uint32))
+
+
+# ------------------------------------------------------------------------------------------------ V3 dynamic quantisation
+QUANT_CASES = [  # T, K, E, H, dtype name, range, smooth
+    (3, 2, 4, 8, "f32", None, False),
+    (60, 3, 12, 40, "f32", (3, 9), True),
+    (64, 8, 128, 4096, "bf16", None, False),       # decode shape
+    (64, 8, 256, 512, "bf16", (32, 64), True),
+    (200, 4, 16, 7168, "bf16", None, False),       # DeepSeek-V3 row width
+    (100, 2, 8, 1000, "f16", None, True),
+    (50, 3, 9, 37, "f16", (2, 7), False),          # odd width: byte path
+    (33, 5, 10, 130, "bf16", None, True),          # width not a multiple of 4
+]
+
+
+@pytest.mark.parametrize("T,K,E,H,dtype_name,rng_,with_smooth", QUANT_CASES)
+def test_v3_dynamic_quant_bit_exact(aclnn, oracle, dev, T, K, E, H, dtype_name, rng_, with_smooth):
+    """int8 rows, scales, indices and counts equal the oracle bit for bit: every step is IEEE arithmetic (abs-max, two
+    divides, a toward-zero narrowing, a halves-away rounding), none of it a library function."""
+    rng = np.random.default_rng(T + H)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype_name]
+    code = {"f32": oracle.DT_F32, "f16": oracle.DT_F16, "bf16": oracle.DT_BF16}[dtype_name]
+    x32 = (rng.standard_normal((T, H)) * 3).astype(np.float32)
+    x32[T // 2] = 0
+    xt = torch.from_numpy(x32).to(tdt)
+    bits = xt.numpy() if dtype_name == "f32" else xt.view(torch.int16).numpy().view(np.uint16)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    start, end = (0, E) if rng_ is None else rng_
+    smooth = (rng.random((end - start, H)) + 0.5).astype(np.float32) if with_smooth else None
+    for mode, row_idx_type in ((1, 1), (0, 0), (2, 1)):
+        ex, ri, cnt, es = aclnn.moe_init_routing_v3(xt.to(dev), torch.from_numpy(idx).to(dev),
+                                                    None if smooth is None else torch.from_numpy(smooth).to(dev),
+                                                    expert_num=E, expert_tokens_num_type=mode, quant_mode=1,
+                                                    active_expert_range=rng_, row_idx_type=row_idx_type)
+        torch.cuda.synchronize()
+        ex_r, ri_r, cnt_r, es_r = oracle.moe_init_routing_v3_quant(bits, idx, smooth, E, rng_, mode, row_idx_type, dtype=code)
+        assert np.array_equal(ri.cpu().numpy(), ri_r) and np.array_equal(cnt.cpu().numpy(), cnt_r)
+        assert np.array_equal(es.cpu().numpy(), es_r)
+        assert np.array_equal(ex.cpu().numpy(), ex_r)
+
+
+def test_v3_dynamic_quant_feeds_the_gemm(pkg, aclnn, oracle, dev):
+    """bf16 activations -> V3 with quantMode 1 gives the int8 rows and scales the SwiGLU GEMM operator consumes."""
+    cfg = pkg.synth.config(0)
+    rng = np.random.default_rng(1)
+    x = torch.from_numpy(rng.standard_normal((cfg.tokens, cfg.hidden)).astype(np.float32)).to(torch.bfloat16).to(dev)
+    idx, _ = pkg.synth.make_routing(cfg, seed=0)
+    w13, w13s, _, _ = pkg.synth.make_weights(cfg, dev, seed=0)
+    ex, ri, cum, es = aclnn.moe_init_routing_v3(x, torch.from_numpy(idx).to(dev), None, expert_num=cfg.experts,
+                                                expert_tokens_num_type=0, quant_mode=1)
+    h, hs = aclnn.grouped_matmul_swiglu_quant(ex, w13.transpose(1, 2), cum, w13s, es)
+    torch.cuda.synchronize()
+    h_r, hs_r = oracle.grouped_matmul_swiglu_quant(ex.cpu().numpy(), w13.cpu().numpy(), w13s.cpu().numpy(), es.cpu().numpy(),
+                                                   cum.cpu().numpy(), w_trans=True)
+    assert np.abs(h.cpu().numpy().astype(np.int32) - h_r.astype(np.int32)).max() <= 1
+    np.testing.assert_allclose(hs.cpu().numpy(), hs_r, rtol=1e-2)

@@ -171,3 +171,61 @@ def test_v3_reference_example_literal(oracle):
     assert cnt.tolist() == [3, 3, 3, 3]
     assert np.array_equal(ex[:, 0], np.array([0.1, 0.2, 0.3, 0.1, 0.2, 0.3, 0.1, 0.2, 0.3, 0.1, 0.2, 0.3], np.float32))
     assert np.array_equal(es, scale[[0, 1, 2] * 4])
+
+
+# ------------------------------------------------------------------------------------------------ V3 dynamic quantisation
+def _trunc_to_half_numpy(v):
+    """fp32 -> fp16 toward zero through numpy: nearest, then one step toward zero where nearest overshot."""
+    h = v.astype(np.float16)
+    over = np.abs(h.astype(np.float32)) > np.abs(v)
+    h = np.where(over, np.nextafter(h, np.float16(0)), h)
+    return h.astype(np.float32)
+
+
+def test_half_truncation_matches_numpy(oracle):
+    rng = np.random.default_rng(2)
+    v = np.concatenate([rng.uniform(-130, 130, 300000), rng.standard_normal(100000) * 1e-3,
+                        rng.standard_normal(50000) * 1e-6, np.arange(-128, 129) + 0.5, np.arange(-128, 129)]).astype(np.float32)
+    assert np.array_equal(oracle.f32_to_f16_trunc_value(v), _trunc_to_half_numpy(v))
+
+
+@pytest.mark.parametrize("with_smooth", [False, True])
+@pytest.mark.parametrize("rng_", [None, (3, 9)])
+def test_v3_dynamic_quant_matches_numpy(oracle, with_smooth, rng_):
+    """Restatement of moe_v3_gather_dynamic_quant.h:103-141 in numpy: abs-max / 127, true divide, half toward zero,
+    halves away from zero."""
+    rng = np.random.default_rng(7)
+    T, K, E, H = 60, 3, 12, 40
+    x = (rng.standard_normal((T, H)) * 4).astype(np.float32)
+    x[5] = 0                                                   # an all-zero token
+    x[6, 3] = 1000.0                                           # one dominant element
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    start, end = (0, E) if rng_ is None else rng_
+    smooth = (rng.random((end - start, H)) + 0.5).astype(np.float32) if with_smooth else None
+    ex, ri, cnt, es = oracle.moe_init_routing_v3_quant(x, idx, smooth, E, rng_, 1, 1)
+    _, ri_r, cnt_r, _ = oracle.moe_init_routing_v3(x, idx, None, E, rng_, 1, 1)
+    assert np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r)
+    flat = idx.reshape(-1)
+    for i in range(T * K):
+        d = ri[i]
+        if d < 0:
+            continue
+        v = x[i // K] * (smooth[flat[i] - start] if with_smooth else np.float32(1))
+        v = v.astype(np.float32)
+        mx = np.abs(v).max()
+        s = np.float32(mx) / np.float32(127.0)
+        assert es[d] == s
+        if mx == 0:
+            assert not ex[d].any()
+            continue
+        h = _trunc_to_half_numpy((v / s).astype(np.float32))
+        want = (np.sign(h) * np.floor(np.abs(h) + 0.5)).astype(np.int8)
+        assert np.array_equal(ex[d], want), i
+        assert np.abs(ex[d].astype(np.int32)).max() == 127
+        assert np.abs(ex[d].astype(np.float32) * s - v).max() <= s * (0.5 + 1 / 16 + 1e-3)
+    routed = (ri >= 0).sum()
+    assert not ex[routed:].any() and not es[routed:].any()
+    # gather-type index and the other count modes reuse the routing of the unquantised operator
+    ex0, ri0, cnt0, es0 = oracle.moe_init_routing_v3_quant(x, idx, smooth, E, rng_, 2, 0)
+    _, ri0_r, cnt0_r, _ = oracle.moe_init_routing_v3(x, idx, None, E, rng_, 2, 0)
+    assert np.array_equal(ri0, ri0_r) and np.array_equal(cnt0, cnt0_r) and np.array_equal(ex0, ex) and np.array_equal(es0, es)
