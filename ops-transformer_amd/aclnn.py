@@ -65,10 +65,17 @@ _PHASE1_SIGNATURES = {
         [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulV5GetWorkspaceSize":
         [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulFinalizeRoutingV3GetWorkspaceSize":
+        [_VP] * 12 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulFinalizeRoutingV2GetWorkspaceSize":
+        [_VP] * 12 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulFinalizeRoutingGetWorkspaceSize":
+        [_VP] * 9 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _U64P, _VPP],
     "aclnnMoeFinalizeRoutingV2GetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _U64P, _VPP],
 }
-_PHASE2 = ["aclnnMoeGatingTopKSoftmaxV2", "aclnnMoeInitRoutingV2", "aclnnMoeInitRoutingV3", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
+_PHASE2 = ["aclnnGroupedMatmulFinalizeRouting", "aclnnGroupedMatmulFinalizeRoutingV2", "aclnnGroupedMatmulFinalizeRoutingV3",
+           "aclnnMoeGatingTopKSoftmaxV2", "aclnnMoeInitRoutingV2", "aclnnMoeInitRoutingV3", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
            "aclnnMoeFinalizeRoutingV2"]
 
 
@@ -363,6 +370,34 @@ def grouped_matmul_v4(x, weight, bias=None, scale=None, offset=None, antiquant_s
 def grouped_matmul_v5(x, weight, tuning_config=(), **kwargs):
     """aclnnGroupedMatmulV5: grouped_matmul_v4 plus the tuning hint (an empty list means "no hint")."""
     return grouped_matmul_v4(x, weight, tuning_config=list(tuning_config), **kwargs)
+
+
+def grouped_matmul_finalize_routing(x, weight, scale, row_index, batch, group_list, group_list_type=1, bias=None,
+                                    per_token_scale=None, logit=None, shared_input=None, shared_input_weight=1.0,
+                                    shared_input_offset=0, tuning_config=None, out=None, workspace=None, version=3):
+    """aclnnGroupedMatmulFinalizeRouting (version 1), V2 or V3: int8 grouped matmul fused with the weighted combine.
+    weight is the [E, K, N] view; returns out fp32 [batch, N]."""
+    dev = x.device
+    N = weight.shape[2]
+    if out is None:
+        out = torch.empty((batch, N), dtype=torch.float32, device=dev)
+    h = _Handles()
+    try:
+        head = [h.tensor(x), h.tensor(weight), h.tensor(scale), h.tensor(bias)]
+        tail = [h.tensor(per_token_scale), h.tensor(group_list), h.tensor(shared_input), h.tensor(logit), h.tensor(row_index),
+                0, float(shared_input_weight), int(shared_input_offset), False, False, int(group_list_type)]
+        if version == 1:
+            api, args = "aclnnGroupedMatmulFinalizeRouting", head + tail + [h.tensor(out)]
+        elif version == 2:
+            api, args = "aclnnGroupedMatmulFinalizeRoutingV2", head + [None, None, None] + tail + [h.tensor(out)]
+        else:
+            api = "aclnnGroupedMatmulFinalizeRoutingV3"
+            args = head + [None, None, None] + tail + [None if tuning_config is None else h.int_array(list(tuning_config)),
+                                                         h.tensor(out)]
+        _run_two_phase(api, args, dev, workspace)
+    finally:
+        h.close()
+    return out
 
 
 def moe_finalize_routing_v2(expanded_x, expanded_row_idx, x1=None, x2=None, bias=None, scales=None, expert_idx=None,

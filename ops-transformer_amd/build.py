@@ -25,6 +25,7 @@ SOURCES = [
     "grouped_gemm_i8.hip",
     "grouped_matmul_swiglu_quant.hip",
     "grouped_matmul_v4.hip",
+    "grouped_matmul_finalize_routing.hip",
     "moe_finalize_routing_v2.hip",
     "calibration_copy.hip",
 ]

@@ -34,6 +34,15 @@ struct Problem {
     const void* scale = nullptr;     // [groups, N] per output channel
     int scaleDtype = 0;
     const float* rowScale = nullptr; // [M] per token, may be null for kDequant
+    // kDequant with fp32 output only: scatter-add instead of store.  Row r of the result is added (atomically, fp32) to
+    // out[combineIndex[r], :] when the index lies in [0, combineRows); with a bias, combineWeight[r] * bias[e, c] is
+    // added to the value first.  `out` is then [combineRows, N] and must hold its initial value before the launch.
+    const void* combineIndex = nullptr;  // [M] int64 or int32
+    bool combineIndexIsInt64 = true;
+    int64_t combineRows = 0;
+    const float* combineWeight = nullptr;  // [M], used with bias only
+    const void* bias = nullptr;            // [groups, N]
+    int biasDtype = 0;
     // kSwiglu only
     int8_t* quantOut = nullptr;      // [M, N/2]
     float* quantScaleOut = nullptr;  // [M]

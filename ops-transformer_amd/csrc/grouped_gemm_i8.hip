@@ -156,6 +156,13 @@ struct KernelArgs {
     const float* rowScale;
     float* sOut;
     float* rowMax;  // [tilesN][M] partial max |S| per n-tile
+    // scatter-add mode of the fp32 kDequant epilogue (Problem::combineIndex)
+    const void* combineIndex;
+    int32_t combineIndexIsInt64;
+    int32_t combineRows;
+    const float* combineWeight;
+    const void* bias;
+    int32_t biasDtype;
 };
 
 // One output tile of one group, decoded from the scheduling table (all fields are wave-uniform).
@@ -238,6 +245,11 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
             if (valid0) sc0 = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + n0, a.scaleDtype);
             if (valid1) sc1 = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + n0 + 32, a.scaleDtype);
         }
+        float bias0 = 0.0f, bias1 = 0.0f;
+        if (kEpi == Epilogue::kDequant && a.bias != nullptr) {
+            if (valid0) bias0 = LoadScale(a.bias, static_cast<int64_t>(group) * a.N + n0, a.biasDtype);
+            if (valid1) bias1 = LoadScale(a.bias, static_cast<int64_t>(group) * a.N + n0 + 32, a.biasDtype);
+        }
         // 16-bit outputs: a lane holds one column of each block, i.e. 2-byte pieces 64 bytes apart.  Neighbouring lanes
         // swap one value so that an even lane owns columns (c, c+1) of block 0 and the odd lane next to it the same pair
         // of block 1; every lane then stores one aligned 32-bit word and a half-wave covers a whole 128-byte row segment.
@@ -295,6 +307,22 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                     y1 = __fmul_rn(y1, rs);
                 }
                 if (a.outDtype == 0) {
+                    if (a.combineIndex != nullptr) {
+                        if (r >= rows) continue;
+                        const int64_t src = rowBase + r;
+                        const int64_t dst = a.combineIndexIsInt64 ? static_cast<const int64_t*>(a.combineIndex)[src]
+                                                                  : static_cast<const int32_t*>(a.combineIndex)[src];
+                        if (dst < 0 || dst >= a.combineRows) continue;
+                        if (a.bias != nullptr) {
+                            const float wgt = a.combineWeight != nullptr ? a.combineWeight[src] : 1.0f;
+                            y0 = __fadd_rn(y0, __fmul_rn(wgt, bias0));
+                            y1 = __fadd_rn(y1, __fmul_rn(wgt, bias1));
+                        }
+                        float* const dstRow = static_cast<float*>(a.out) + dst * a.N;
+                        if (valid0) unsafeAtomicAdd(dstRow + n0, y0);
+                        if (valid1) unsafeAtomicAdd(dstRow + n0 + 32, y1);
+                        continue;
+                    }
                     if (r < rows && valid0) static_cast<float*>(a.out)[rowOff + n0] = y0;
                     if (r < rows && valid1) static_cast<float*>(a.out)[rowOff + n0 + 32] = y1;
                     continue;
@@ -1351,7 +1379,8 @@ Plan MakePlan(const Problem& p) {
     {
         // read at plan time (not cached) so that one process can plan either way
         const char* env = std::getenv("OPAPI_GEMM_PATH");
-        plan.regPath = StreamOk(p) && plan.tileM <= 192 && env != nullptr && std::string(env) == "reg";
+        plan.regPath = StreamOk(p) && plan.tileM <= 192 && p.combineIndex == nullptr && env != nullptr &&
+                       std::string(env) == "reg";
     }
     plan.wavesM = plan.tileM >= 64 && StreamOk(p) ? 2 : 1;
     plan.subTilesM = (plan.tileM / 32 + plan.wavesM - 1) / plan.wavesM;
@@ -1417,12 +1446,19 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.rowScale = p.rowScale;
     ka.sOut = sBuf;
     ka.rowMax = rowMax;
+    ka.combineIndex = p.combineIndex;
+    ka.combineIndexIsInt64 = p.combineIndexIsInt64 ? 1 : 0;
+    ka.combineRows = static_cast<int32_t>(p.combineRows);
+    ka.combineWeight = p.combineWeight;
+    ka.bias = p.bias;
+    ka.biasDtype = p.biasDtype;
 
     hipError_t e = hipSuccess;
     if (p.K > 0) {
         const bool fast = StreamOk(p);
         opapi::KernelTimer timer(p.epilogue == Epilogue::kSwiglu ? "gmm_swiglu"
-                                 : p.epilogue == Epilogue::kDequant ? "gmm_dequant" : "gmm_int32", stream);
+                                 : p.epilogue != Epilogue::kDequant ? "gmm_int32"
+                                 : p.combineIndex != nullptr ? "gmm_combine" : "gmm_dequant", stream);
         switch (p.epilogue) {
             case Epilogue::kInt32:
                 e = fast ? LaunchFast<Epilogue::kInt32>(plan, ka, sched, stream)

@@ -12,6 +12,10 @@ Glue between the operators:
     arrangement expandedRowIdx[n*K + k] = destination.
 ``routing="v2"`` keeps the older chain: MoeInitRoutingV2 on the rows plus a second MoeInitRoutingV2 call on the
 [T, 1] scale column, int32 cumsum.
+``fused_combine=True`` replaces the last two operators by aclnnGroupedMatmulFinalizeRoutingV3 (down projection with
+the weighted combine as scatter-add): routing then emits the gather-type index (rowIdxType 0), from which the glue
+derives the fused operator's rowIndex (destination token = source // K) and logit (the top-k weight of that source);
+the result is fp32 [T, H], and the order of the K additions per token is not fixed.
 """
 import torch
 
@@ -29,9 +33,11 @@ class MoeFfnW8A8:
     The operators see the reference layout [E, K, N] through transposed views of this storage.
     """
 
-    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v3"):
+    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v3", fused_combine=False):
         assert routing in ("v2", "v3")
+        assert not (fused_combine and routing != "v3")
         self.routing = routing
+        self.fused_combine = fused_combine
         assert w13.dtype == torch.int8 and w2.dtype == torch.int8
         self.w13_view = w13.transpose(1, 2)  # [E, H, 2I]
         self.w2_view = w2.transpose(1, 2)    # [E, I, H]
@@ -56,7 +62,7 @@ class MoeFfnW8A8:
         self.h = torch.empty((M, I), dtype=torch.int8, device=dev)
         self.h_scale = torch.empty((M,), dtype=torch.float32, device=dev)
         self.y = torch.empty((M, H), dtype=self.out_dtype, device=dev)
-        self.out = torch.empty((T, H), dtype=self.out_dtype, device=dev)
+        self.out = torch.empty((T, H), dtype=torch.float32 if self.fused_combine else self.out_dtype, device=dev)
         # one workspace shared by the chain; it grows to the largest phase-1 request on the first pass
         self.workspace = aclnn.Workspace()
         self._buf_key = (T, K)
@@ -68,7 +74,7 @@ class MoeFfnW8A8:
         E = self.num_experts
         if self.routing == "v3":
             aclnn.moe_init_routing_v3(xq, topk_idx, x_scale, expert_num=E, expert_tokens_num_type=0, quant_mode=-1,
-                                      row_idx_type=1,
+                                      row_idx_type=0 if self.fused_combine else 1,
                                       out=(self.expanded_x, self.expanded_row_idx, self.cumsum, self.expanded_scale),
                                       workspace=self.workspace)
         else:
@@ -81,6 +87,13 @@ class MoeFfnW8A8:
         aclnn.grouped_matmul_swiglu_quant(self.expanded_x, self.w13_view, self.cumsum, self.w13_scale,
                                           self.expanded_scale, out=(self.h, self.h_scale),
                                           workspace=self.workspace)
+        if self.fused_combine:
+            source = self.expanded_row_idx.long()                       # expanded row -> flat (token, k) position
+            logit = topk_weight.reshape(-1).float()[source]
+            aclnn.grouped_matmul_finalize_routing(self.h, self.w2_view, self.w2_scale, source // K, T, self.cumsum,
+                                                  group_list_type=0, per_token_scale=self.h_scale, logit=logit,
+                                                  out=self.out, workspace=self.workspace)
+            return self.out
         aclnn.grouped_matmul_v4([self.h], [self.w2_view], scale=[self.w2_scale], per_token_scale=[self.h_scale],
                                 group_list=self.cumsum, split_item=3, group_type=0, group_list_type=0, act_type=0,
                                 out=[self.y], workspace=self.workspace)

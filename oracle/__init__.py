@@ -269,6 +269,27 @@ def grouped_matmul_dequant(x, w, scale, per_token, group_list, list_type=0, w_tr
     return out
 
 
+def grouped_matmul_finalize_routing(x, w, scale, row_index, batch, group_list, list_type=1, w_trans=False, bias=None,
+                                    per_token=None, logit=None, shared=None, shared_dtype=DT_BF16, shared_offset=0,
+                                    shared_weight=1.0, scale_dtype=DT_F32, bias_dtype=DT_BF16):
+    """GroupedMatmulFinalizeRouting with INT8 weights.  scale / bias: fp32 arrays or uint16 bit patterns per their dtype;
+    shared: uint16 bit patterns [rows, N].  Returns out fp32 [batch, N]."""
+    x, w, M, K, N, gl, _, _ = _gemm_common(x, w, w_trans, group_list, None)
+    sc = _c(scale, np.float32 if scale_dtype == DT_F32 else np.uint16)
+    bs = None if bias is None else _c(bias, np.float32 if bias_dtype == DT_F32 else np.uint16)
+    pt = None if per_token is None else _c(per_token, np.float32)
+    lg = None if logit is None else _c(logit, np.float32)
+    ri = _c(row_index, np.int64)
+    sh = None if shared is None else _c(shared, np.uint16)
+    out = np.empty((batch, N), np.float32)
+    lib().oracle_grouped_matmul_finalize_routing(
+        _p(x), _p(w), ctypes.c_int(int(w_trans)), _p(sc), ctypes.c_int(scale_dtype), _p(bs), ctypes.c_int(bias_dtype), _p(pt),
+        _p(lg), _p(ri), ctypes.c_int64(M), ctypes.c_int64(K), ctypes.c_int64(N), ctypes.c_int64(gl.shape[0]), _p(gl),
+        ctypes.c_int64(list_type), _p(sh), ctypes.c_int(shared_dtype), ctypes.c_int64(0 if sh is None else sh.shape[0]),
+        ctypes.c_int64(shared_offset), ctypes.c_float(shared_weight), ctypes.c_int64(batch), _p(out))
+    return out
+
+
 # ----------------------------------------------------------------------------------------------- finalize
 def moe_finalize_routing_v2(expanded_x, expanded_row_idx, x1=None, x2=None, bias=None, scales=None, expert_idx=None,
                             drop_pad_mode=0, dtype=DT_F32, scale_dtype=None):

@@ -513,6 +513,53 @@ ORACLE_API void oracle_grouped_matmul_dequant(const int8_t* x, const int8_t* w, 
     free(begin);
 }
 
+/* GroupedMatmulFinalizeRouting with INT8 weights (gmm/grouped_matmul_finalize_routing/op_kernel/
+ * grouped_matmul_finalize_routing.h): out [batch, N] fp32 starts at zero, rows [sharedOffset, sharedOffset + sharedRows)
+ * at float(shared) * sharedWeight (:217-254); every row r of x in group e adds
+ *   (float(acc[r, c]) * scale[e, c]) * (perToken[r] * logit[r])  [+ logit[r] * float(bias[e, c])]        (:390-417, :458-495)
+ * to out[rowIndex[r], c] (:321-342).  The reference adds with fp32 atomics in no fixed order; here rows are added in
+ * ascending r.  perToken, logit, bias, shared may be NULL (factor 1 / none). */
+ORACLE_API void oracle_grouped_matmul_finalize_routing(const int8_t* x, const int8_t* w, int wTrans, const void* scale,
+                                                       int scaleDtype, const void* bias, int biasDtype, const float* perToken,
+                                                       const float* logit, const int64_t* rowIndex, int64_t M, int64_t K,
+                                                       int64_t N, int64_t G, const int64_t* groupList, int64_t listType,
+                                                       const uint16_t* shared, int sharedDtype, int64_t sharedRows,
+                                                       int64_t sharedOffset, float sharedWeight, int64_t batch, float* out) {
+    int64_t* begin = (int64_t*)malloc(sizeof(int64_t) * (size_t)(G + 1));
+    group_bounds(groupList, G, listType, begin);
+    for (int64_t i = 0; i < batch * N; i++) out[i] = 0.f;
+    for (int64_t j = 0; j < sharedRows; j++) {
+        for (int64_t c = 0; c < N; c++) out[(sharedOffset + j) * N + c] = load_as_f32(shared, j * N + c, sharedDtype) * sharedWeight;
+    }
+    float* contrib = (float*)malloc(sizeof(float) * (size_t)(M > 0 ? M : 1) * (size_t)N);
+#pragma omp parallel
+    {
+        int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)N);
+#pragma omp for schedule(dynamic, 4)
+        for (int64_t r = 0; r < M; r++) {
+            const int64_t e = find_group(begin, G, r);
+            if (e < 0) { for (int64_t c = 0; c < N; c++) contrib[r * N + c] = 0.f; continue; }
+            gemm_row_i32(x + r * K, w + e * K * N, wTrans, K, N, acc);
+            float factor = perToken ? perToken[r] : 1.0f;
+            if (logit) factor = factor * logit[r];
+            for (int64_t c = 0; c < N; c++) {
+                float v = ((float)acc[c] * load_as_f32(scale, e * N + c, scaleDtype)) * factor;
+                if (bias) v = v + (logit ? logit[r] : 1.0f) * load_as_f32(bias, e * N + c, biasDtype);
+                contrib[r * N + c] = v;
+            }
+        }
+        free(acc);
+    }
+    for (int64_t r = 0; r < M; r++) {
+        if (find_group(begin, G, r) < 0) continue;
+        const int64_t d = rowIndex[r];
+        if (d < 0 || d >= batch) continue;
+        for (int64_t c = 0; c < N; c++) out[d * N + c] += contrib[r * N + c];
+    }
+    free(contrib);
+    free(begin);
+}
+
 /* ------------------------------------------------------------------------------------------------ finalize */
 
 /*

@@ -32,6 +32,9 @@ def test_headers_declare_the_expected_entry_points():
     for required in ["aclnnMoeInitRoutingV2GetWorkspaceSize", "aclnnMoeInitRoutingV2",
                      "aclnnMoeInitRoutingV3GetWorkspaceSize", "aclnnMoeInitRoutingV3",
                      "aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize", "aclnnMoeGatingTopKSoftmaxV2",
+                     "aclnnGroupedMatmulFinalizeRoutingGetWorkspaceSize", "aclnnGroupedMatmulFinalizeRouting",
+                     "aclnnGroupedMatmulFinalizeRoutingV2GetWorkspaceSize", "aclnnGroupedMatmulFinalizeRoutingV2",
+                     "aclnnGroupedMatmulFinalizeRoutingV3GetWorkspaceSize", "aclnnGroupedMatmulFinalizeRoutingV3",
                      "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize", "aclnnGroupedMatmulSwigluQuant",
                      "aclnnGroupedMatmulV4GetWorkspaceSize", "aclnnGroupedMatmulV4",
                      "aclnnGroupedMatmulV5GetWorkspaceSize", "aclnnGroupedMatmulV5",
@@ -378,6 +381,89 @@ def test_gmm_v5_takes_a_tuning_hint(aclnn):
     args = args[:16] + [None] + args[16:]
     code, msg = _status(aclnn, "aclnnGroupedMatmulV5", args)
     assert code == INVALID and "groupType 0" in msg
+
+
+# ------------------------------------------------------------------------------------------------ fused combine
+def _combine_args(aclnn, M=64, K=256, N=128, E=4, batch=16, version=3, **over):
+    x = T(aclnn, (M, K), over.get("x_dtype", I8))
+    w = T(aclnn, over.get("w_shape", (E, K, N)), over.get("w_dtype", I8), fmt=over.get("w_fmt", 2))
+    scale = T(aclnn, over.get("scale_shape", (E, N)), over.get("scale_dtype", F32))
+    bias = T(aclnn, over.get("bias_shape", (E, N)), over.get("bias_dtype", BF16)) if over.get("with_bias", True) else None
+    pt = T(aclnn, over.get("pt_shape", (M,)), F32) if over.get("with_pt", True) else None
+    gl = T(aclnn, (over.get("gl_len", E),), over.get("gl_dtype", I64))
+    shared = T(aclnn, over.get("shared_shape", (4, N)), over.get("shared_dtype", BF16)) if over.get("with_shared", True) else None
+    logit = T(aclnn, over.get("logit_shape", (M,)), F32) if over.get("with_logit", True) else None
+    ri = T(aclnn, over.get("ri_shape", (M,)), over.get("ri_dtype", I64))
+    out = T(aclnn, over.get("out_shape", (batch, N)), over.get("out_dtype", F32))
+    head = [x.h, w.h, scale.h, bias.h if bias else None]
+    tail = [pt.h if pt else None, gl.h, shared.h if shared else None, logit.h if logit else None, ri.h,
+            over.get("dtype", 0), 1.0, over.get("shared_offset", 0), over.get("tx", False), over.get("tw", False),
+            over.get("group_list_type", 1)]
+    extra = [over.get("offset"), over.get("anti"), None]
+    if version == 1:
+        return "aclnnGroupedMatmulFinalizeRouting", head + tail + [out.h]
+    if version == 2:
+        return "aclnnGroupedMatmulFinalizeRoutingV2", head + extra + tail + [out.h]
+    tuning = over.get("tuning")
+    arr = None if tuning is None else aclnn.lib().aclCreateIntArray((ctypes.c_int64 * len(tuning))(*tuning), len(tuning))
+    return "aclnnGroupedMatmulFinalizeRoutingV3", head + extra + tail + [arr, out.h]
+
+
+def test_combine_valid(aclnn):
+    for kw in [dict(), dict(version=1), dict(version=2), dict(scale_dtype=BF16), dict(scale_shape=(4, 1, 128)),
+               dict(with_bias=False, with_pt=False, with_shared=False, with_logit=False), dict(bias_dtype=F32),
+               dict(ri_dtype=I32), dict(gl_dtype=I32), dict(group_list_type=0), dict(shared_dtype=F16, shared_offset=12),
+               dict(tuning=[16]), dict(batch=64), dict(batch=0, with_shared=False)]:
+        api, args = _combine_args(aclnn, **kw)
+        code, ws = _status(aclnn, api, args)
+        assert code == 0, (kw, ws)
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    # rules of gmm/grouped_matmul_finalize_routing/op_host/op_api/aclnn_grouped_matmul_finalize_routing.cpp
+    (dict(dtype=1), "dtype must be 0"),
+    (dict(tx=True), "transpose should be false"),
+    (dict(tw=True), "transpose should be false"),
+    (dict(w_dtype=I32, w_shape=(4, 256, 16)), "INT4 weights"),
+    (dict(w_fmt=29), "format should be ND"),
+    (dict(x_dtype=BF16), "x1 must be INT8"),
+    (dict(scale_dtype=I64), "scale must be FLOAT or BF16"),
+    (dict(scale_shape=(3, 128)), "Scale fisrt dim should equal to weight EDim 4, but actual is 3"),
+    (dict(bias_shape=(4, 127)), "bias's dim value should be (e, n)"),
+    (dict(pt_shape=(63,)), "pertokenScale fisrt dim should equal to x MDim 64"),
+    (dict(gl_len=5), "groupList fisrt dim should equal to weight EDim 4"),
+    (dict(logit_shape=(65,)), "logit fisrt dim should equal to x MDim 64"),
+    (dict(ri_shape=(60,)), "rowIndex fisrt dim should equal to x MDim 64"),
+    (dict(ri_dtype=F32), "rowIndex must be INT64 or INT32"),
+    (dict(batch=65), "Out 1st dim should be less than or equal to x MDim"),
+    (dict(out_shape=(16, 64)), "Out 2nd dim"),
+    (dict(out_dtype=BF16), "out must be FLOAT"),
+    (dict(shared_offset=-1), "sharedInputOffset should bigger than or equal to 0"),
+    (dict(shared_offset=13), "exceeds outputBS 16"),
+    (dict(shared_shape=(17, 128)), "less than or equal to outputBS 16"),
+    (dict(group_list_type=2), "groupListType should be 0 or 1"),
+    (dict(w_shape=(4, 255, 128)), "k dim"),
+    (dict(tuning=[-1]), "Invalid tuningConfigOptional (-1)"),
+    (dict(version=2, offset=1), "offset belongs to the INT4 case"),
+])
+def test_combine_invalid(aclnn, kw, fragment):
+    if kw.get("offset") == 1:
+        kw = dict(kw, offset=T(aclnn, (4, 1, 128), F32).h)
+    api, args = _combine_args(aclnn, **kw)
+    code, msg = _status(aclnn, api, args)
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_combine_nulls(aclnn):
+    for pos in (0, 1, 2):
+        api, args = _combine_args(aclnn)
+        args[pos] = None
+        assert _status(aclnn, api, args)[0] == NULLPTR, pos
+    api, args = _combine_args(aclnn)
+    args[-1] = None                                             # out
+    assert _status(aclnn, api, args)[0] == NULLPTR
+    api, args = _combine_args(aclnn, version=2, anti=T(aclnn, (4, 128), F32).h)   # antiquant arguments are not enabled
+    assert _status(aclnn, api, args)[0] == NULLPTR
 
 
 def test_reference_examples_compile_and_link_unmodified():

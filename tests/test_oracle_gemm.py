@@ -148,3 +148,57 @@ def test_swiglu_zero_row_is_defined(oracle):
     y, ys = oracle.grouped_matmul_swiglu_quant(x, w, np.ones((1, 8), np.float32), np.ones(2, np.float32),
                                                np.array([2], np.int64))
     assert (y == 0).all() and (ys == 0).all()
+
+
+# ------------------------------------------------------------------------------------------------ fused combine
+def test_grouped_matmul_finalize_routing_matches_float64(oracle):
+    """GroupedMatmulFinalizeRouting: float64 numpy restatement (exact matmul per group, contributions scattered with
+    np.add.at).  fp32 against float64: a sum of up to `top_k` products, tolerance 1e-5 of the largest term."""
+    rng = np.random.default_rng(4)
+    M, K, N, E, batch, topk = 96, 128, 40, 5, 24, 4
+    x, w, cumsum = _problem(rng, M, K, N, E)
+    counts = np.diff(np.concatenate([[0], cumsum])).astype(np.int64)
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    bias32 = rng.standard_normal((E, N)).astype(np.float32)
+    bias_bits = oracle.f32_to_bf16_bits(bias32)
+    bias = oracle.bf16_bits_to_f32(bias_bits)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    logit = rng.random(M).astype(np.float32)
+    row_index = np.repeat(np.arange(batch), topk)
+    rng.shuffle(row_index)
+    shared_bits = oracle.f32_to_bf16_bits(rng.standard_normal((6, N)).astype(np.float32))
+    shared = oracle.bf16_bits_to_f32(shared_bits)
+    got = oracle.grouped_matmul_finalize_routing(x, w, scale, row_index, batch, counts, list_type=1, bias=bias_bits,
+                                                 per_token=pt, logit=logit, shared=shared_bits, shared_offset=10,
+                                                 shared_weight=0.5)
+    acc = _f64_grouped(x, w, cumsum)
+    group_of = np.searchsorted(cumsum, np.arange(M), side="right")
+    contrib = acc * scale[group_of].astype(np.float64) * (pt.astype(np.float64) * logit)[:, None] \
+        + logit[:, None].astype(np.float64) * bias[group_of]
+    want = np.zeros((batch, N))
+    want[10:16] = shared.astype(np.float64) * 0.5
+    np.add.at(want, row_index, contrib)
+    scale_of_terms = np.abs(contrib).max()
+    assert np.abs(got - want).max() <= 1e-5 * scale_of_terms
+    # cumsum list, transposed storage, no optional inputs: a plain scatter of the dequantised rows
+    wt = np.ascontiguousarray(w.transpose(0, 2, 1))
+    got2 = oracle.grouped_matmul_finalize_routing(x, wt, scale, row_index, batch, cumsum, list_type=0, w_trans=True)
+    want2 = np.zeros((batch, N))
+    np.add.at(want2, row_index, acc * scale[group_of].astype(np.float64))
+    assert np.abs(got2 - want2).max() <= 1e-5 * np.abs(acc * scale[group_of]).max()
+    # rows beyond the last group and indices outside [0, batch) contribute nothing
+    short = cumsum.copy()
+    short[-1] = short[-2]
+    bad = row_index.copy()
+    bad[:3] = [-1, batch, batch + 5]
+    got3 = oracle.grouped_matmul_finalize_routing(x, w, scale, bad, batch, short, list_type=0)
+    keep = (np.arange(M) < short[-1]) & (bad >= 0) & (bad < batch)
+    want3 = np.zeros((batch, N))
+    np.add.at(want3, bad[keep], (acc * scale[group_of.clip(max=E - 1)].astype(np.float64))[keep])
+    assert np.abs(got3 - want3).max() <= 1e-5 * np.abs(acc).max() * scale.max()
+    # equivalence with the unfused pair: down projection to fp32, then a weighted scatter
+    y = oracle.grouped_matmul_dequant(x, w, scale, pt, cumsum, out_dtype=oracle.DT_F32)
+    want4 = np.zeros((batch, N))
+    np.add.at(want4, row_index, y.astype(np.float64) * logit[:, None])
+    got4 = oracle.grouped_matmul_finalize_routing(x, w, scale, row_index, batch, cumsum, list_type=0, per_token=pt, logit=logit)
+    assert np.abs(got4 - want4).max() <= 1e-5 * np.abs(y).max()
