@@ -1,6 +1,7 @@
 """Benchmark of the quantized MoE expert-FFN path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline] [--calibration-copy]
+                    [--fused-combine]
 
 A step is one pass of the path (routing -> gate/up GEMM + SwiGLU + requant -> down GEMM -> finalize) over one batch of
 synthetic tokens whose inputs and expert weights are already resident in HBM.  Prints ONE JSON line: tokens/s for the
@@ -86,6 +87,8 @@ def main():
     ap.add_argument("--config", default="c1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true")
+    ap.add_argument("--fused-combine", action="store_true",
+                    help="end the chain with aclnnGroupedMatmulFinalizeRoutingV3 instead of GroupedMatmulV4 + MoeFinalizeRoutingV2")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (expert parallelism is a design note only); "
@@ -106,7 +109,7 @@ def main():
     idx, wgt = pkg.synth.make_routing(cfg, seed=seed)
     xq, xs = pkg.synth.make_activations(cfg, seed=seed)
     w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=seed)
-    ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s)
+    ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, fused_combine=args.fused_combine)
     d_xq, d_xs = torch.from_numpy(xq).to(dev), torch.from_numpy(xs).to(dev)
     d_idx, d_wgt = torch.from_numpy(idx).to(dev), torch.from_numpy(wgt).to(dev)
 
@@ -175,7 +178,8 @@ def main():
         "config": {"workload": "%s: %d tokens, H=%d, I=%d, E=%d, top-%d, %s routing" % (
             cfg.name, cfg.tokens, cfg.hidden, cfg.inter, cfg.experts, cfg.top_k,
             "Zipf(%.1f)" % cfg.skew if cfg.skew else "uniform random"),
-            "expanded_rows": M, "experts_touched": touched, "weight_layout": "K-contiguous (transposed view)"},
+            "expanded_rows": M, "experts_touched": touched, "weight_layout": "K-contiguous (transposed view)",
+            "chain": "V3 routing, SwiGLU GEMM, " + ("fused down GEMM + combine" if args.fused_combine else "down GEMM, finalize")},
         "end_to_end": {"tops": work["ops"] / (elapsed / args.steps) / 1e12, "gbps": work["bytes"] / (elapsed / args.steps) / 1e9,
                        "mfma_frac": work["ops"] / (elapsed / args.steps) / 1e12 / INT8_PEAK_TOPS,
                        "hbm_frac": work["bytes"] / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,

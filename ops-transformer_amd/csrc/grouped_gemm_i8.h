@@ -13,7 +13,8 @@ enum class Epilogue : int {
     kSwiglu = 2,   // S = swish(C[:, j]) * C[:, j + N/2] with C = (float(acc) * rowScale[r]) * scale[e,c]; S and row max |S| out
 };
 
-enum class GroupListKind : int { kCumsum = 0, kCount = 1 };
+// kSparse: [groups, 2] pairs (expert id, rows) in row order, ended by the first pair without rows.
+enum class GroupListKind : int { kCumsum = 0, kCount = 1, kSparse = 2 };
 
 // Element type codes follow aclDataType: 0 fp32, 1 fp16, 27 bf16, 3 int32.
 struct Problem {
@@ -23,7 +24,7 @@ struct Problem {
     bool wKMajor = true;
     int64_t M = 0, K = 0, N = 0;
     int32_t groups = 0;
-    const void* groupList = nullptr; // device, int64 or int32, cumsum or counts
+    const void* groupList = nullptr; // device, int64 or int32: cumsum or counts [groups], or sparse pairs [groups, 2]
     bool groupListIsInt64 = true;
     GroupListKind groupListKind = GroupListKind::kCumsum;
     int64_t expectedRowsPerGroup = 0; // > 0: caller's hint for the tile height; 0: use M / groups

@@ -61,7 +61,7 @@ struct SchedArgs {
     int32_t* sched;
     int32_t groups;
     int32_t groupListIsInt64;
-    int32_t isCount;
+    int32_t isCount;  // 0 cumsum, 1 counts, 2 sparse (expert id, count) pairs
     int32_t tileM;
     int32_t maxMTiles;
     int64_t M;
@@ -89,7 +89,37 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
     };
     // group boundaries, clamped into [0, M] and made monotonic so that a malformed list cannot push rows out of range
     int64_t begin = 0, end = 0;
-    if (t < a.groups) {
+    if (a.isCount == 2) {
+        // Sparse list [groups, 2]: pair p = (expert id, rows); pairs take consecutive row ranges in list order and the
+        // list ends at the first pair without rows.  The table stays indexed by expert: an expert named by a pair gets
+        // that pair's row range, every other expert none (an expert named twice keeps the later range only).
+        __shared__ int32_t firstEmpty;
+        __shared__ int32_t expertBegin[kMaxGroups], expertEnd[kMaxGroups];
+        if (t == 0) firstEmpty = a.groups;
+        expertBegin[t] = 0;
+        expertEnd[t] = 0;
+        __syncthreads();
+        int64_t key = -1, val = 0;
+        if (t < a.groups) {
+            key = at(2 * t);
+            val = at(2 * t + 1);
+            if (val <= 0) atomicMin(&firstEmpty, t);
+        }
+        __syncthreads();
+        if (t >= firstEmpty) val = 0;
+        val = val > a.M ? a.M : val;
+        const int32_t inc = inclusiveScan(static_cast<int32_t>(val));
+        int64_t pairEnd = inc, pairBegin = inc - val;
+        pairBegin = pairBegin > a.M ? a.M : pairBegin;
+        pairEnd = pairEnd > a.M ? a.M : pairEnd;
+        if (val > 0 && key >= 0 && key < a.groups) {
+            expertBegin[key] = static_cast<int32_t>(pairBegin);
+            expertEnd[key] = static_cast<int32_t>(pairEnd);
+        }
+        __syncthreads();
+        begin = expertBegin[t];
+        end = expertEnd[t];
+    } else if (t < a.groups) {
         if (a.isCount) {
             int64_t c = at(t);
             c = c < 0 ? 0 : (c > a.M ? a.M : c);
@@ -99,7 +129,7 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
             begin = t > 0 ? at(t - 1) : 0;
         }
     }
-    if (a.isCount) {
+    if (a.isCount == 1) {
         const int32_t inc = inclusiveScan(static_cast<int32_t>(end));
         begin = static_cast<int64_t>(inc) - end;
         end = inc;
@@ -109,6 +139,18 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
     const int32_t rows = t < a.groups ? static_cast<int32_t>(end - begin) : 0;
     const int32_t tiles = (rows + a.tileM - 1) / a.tileM;
     const int32_t tileInc = inclusiveScan(tiles);
+    // rows covered by the list: the end of the last group, or with a sparse list the furthest end of any expert
+    int32_t covered = static_cast<int32_t>(end);
+    if (a.isCount == 2) {
+        scan[t] = t < a.groups ? static_cast<int32_t>(end) : 0;
+        __syncthreads();
+        for (int d = 512; d > 0; d >>= 1) {
+            if (t < d) scan[t] = max(scan[t], scan[t + d]);
+            __syncthreads();
+        }
+        covered = scan[0];
+        __syncthreads();
+    }
     int32_t* rowStart = a.sched + 2;
     int32_t* rowCount = rowStart + a.groups;
     int32_t* tilePrefix = rowCount + a.groups;
@@ -118,7 +160,7 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
         tilePrefix[t] = tileInc - tiles;
         if (t == a.groups - 1) {
             tilePrefix[a.groups] = tileInc;
-            a.sched[0] = static_cast<int32_t>(end);
+            a.sched[0] = covered;
             a.sched[1] = tileInc;
         }
     }
@@ -1418,7 +1460,7 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     sa.sched = sched;
     sa.groups = p.groups;
     sa.groupListIsInt64 = p.groupListIsInt64 ? 1 : 0;
-    sa.isCount = p.groupListKind == GroupListKind::kCount ? 1 : 0;
+    sa.isCount = static_cast<int32_t>(p.groupListKind);
     sa.tileM = plan.tileM;
     sa.maxMTiles = plan.maxMTiles;
     sa.M = p.M;

@@ -7,7 +7,8 @@
 //   :339-361   groupList is a 1-D INT64 tensor of at most 1024 entries whose length equals weight.dim0
 //   :556-588   perTokenScale is FLOAT [M]
 //   :642-700   int8 pairing: scale BF16 -> out BF16, scale FLOAT -> out FLOAT16 (per-token), no scale -> out INT32
-//   :1883-1916 groupListType 0/1 (2 = sparse list, not built), actType range
+//   :1883-1916 groupListType 0/1/2 (2 = sparse [e, 2] list of (expert id, rows) pairs, groupType 0 only), actType range
+//   op_kernel/grouped_matmul.h:288-345 how a sparse list is walked (pairs in order, stop at the first empty pair)
 // Widenings of this build: scale FLOAT with out BF16 is accepted; groupList may be INT32.
 // Group boundaries: grouped_matmul_utils.h:243-257.  The arithmetic is in grouped_gemm_i8.hip.
 #include "aclnnop/aclnn_grouped_matmul_v5.h"
@@ -88,10 +89,16 @@ aclnnStatus PlanGroupedMatmul(
         OPAPI_CHECK(actType < END_ACT_TYPE_ENUM, kInvalid, "Activation function only support RELU/GELU_TANH/FASTGELU/SILU.");
     }
     OPAPI_CHECK(groupListType == 0 || groupListType == 1 || groupListType == 2, kInvalid, "groupListType shoule be 0 or 1.");
-    OPAPI_CHECK(groupListType != 2, kInvalid, "groupListType 2 (sparse group list) is not built on this platform.");
-    OPAPI_CHECK(groupListOptional == nullptr || groupListOptional->dims.size() == 1, kInvalid,
-                "When groupList type is tensor, groupList dim only support 1, but now groupList dim is %zu.",
-                groupListOptional ? groupListOptional->dims.size() : size_t(0));
+    const size_t groupListRank = groupListType == 2 ? 2 : 1;
+    OPAPI_CHECK(groupListOptional == nullptr || groupListOptional->dims.size() == groupListRank, kInvalid,
+                "When groupList type is tensor, groupList dim only support 1 or 2(only when groupListType is 2), but now "
+                "groupList dim is %zu, groupListType is %lld.",
+                groupListOptional ? groupListOptional->dims.size() : size_t(0), (long long)groupListType);
+    OPAPI_CHECK(!(groupListType == 2 && groupListOptional != nullptr && groupListOptional->dims[1] != 2), kInvalid,
+                "With groupListType 2 groupList must be [e, 2] pairs of (expert id, rows), got %s",
+                groupListOptional ? ShapeStr(groupListOptional).c_str() : "");
+    OPAPI_CHECK(!(groupListType == 2 && groupType != 0), kInvalid,
+                "When groupListType is 2 only support groupType 0, but get groupType %lld.", (long long)groupType);
 
     // reserved arguments
     OPAPI_CHECK(!Present(activationInputOptional), kInvalid, "activationInputOptional must be nullptr.");
@@ -199,7 +206,8 @@ aclnnStatus PlanGroupedMatmul(
     p.groups = static_cast<int32_t>(groupListLen);
     p.groupList = DataPtr(groupListOptional);
     p.groupListIsInt64 = groupListOptional->dtype == ACL_INT64;
-    p.groupListKind = groupListType == 1 ? gemm::GroupListKind::kCount : gemm::GroupListKind::kCumsum;
+    p.groupListKind = groupListType == 2 ? gemm::GroupListKind::kSparse
+                      : groupListType == 1 ? gemm::GroupListKind::kCount : gemm::GroupListKind::kCumsum;
     p.out = DataPtr(yt);
     p.outDtype = static_cast<int>(yt->dtype);
     if (scale == nullptr) {

@@ -310,7 +310,7 @@ def _gmm_args(aclnn, M=64, K=256, N=128, E=4, scale_dtype=F32, out_dtype=BF16, p
     w = _tl(aclnn, [T(aclnn, over.get("w_shape", (E, K, N)), I8)])
     scale = _tl(aclnn, [T(aclnn, (E, N), scale_dtype)]) if scale_dtype is not None else None
     pt = _tl(aclnn, [T(aclnn, over.get("pt_shape", (M,)), F32)]) if per_token else None
-    gl = T(aclnn, (over.get("gl_len", E),), over.get("gl_dtype", I64))
+    gl = T(aclnn, over.get("gl_shape", (over.get("gl_len", E),)), over.get("gl_dtype", I64))
     out = _tl(aclnn, [T(aclnn, over.get("out_shape", (M, N)), out_dtype)])
     args = [x, w, over.get("bias"), scale, over.get("offset"), None, None, pt, gl.h if over.get("with_gl", True) else None,
             over.get("act_in"), None, None, over.get("split_item", 3), over.get("group_type", 0),
@@ -320,7 +320,8 @@ def _gmm_args(aclnn, M=64, K=256, N=128, E=4, scale_dtype=F32, out_dtype=BF16, p
 
 def test_gmm_valid(aclnn):
     for kw in [dict(), dict(scale_dtype=BF16), dict(out_dtype=F16), dict(scale_dtype=None, out_dtype=I32, per_token=False),
-               dict(group_list_type=1), dict(split_item=2), dict(gl_dtype=I32), dict(per_token=False)]:
+               dict(group_list_type=1), dict(split_item=2), dict(gl_dtype=I32), dict(per_token=False),
+               dict(group_list_type=2, gl_shape=(4, 2))]:
         code, ws = _status(aclnn, "aclnnGroupedMatmulV4", _gmm_args(aclnn, **kw))
         assert code == 0, (kw, ws)
 
@@ -338,7 +339,9 @@ def test_gmm_empty_optional_means_absent(aclnn):
     (dict(scale_dtype=None, out_dtype=BF16, per_token=False), "must be INT32"),
     (dict(group_type=2), "groupType 0"),
     (dict(split_item=0), "splitItem 2 or 3"),
-    (dict(group_list_type=2), "sparse"),
+    (dict(group_list_type=2), "groupList dim only support 1 or 2(only when groupListType is 2)"),
+    (dict(group_list_type=2, gl_shape=(4, 3)), "[e, 2] pairs"),
+    (dict(group_list_type=1, gl_shape=(4, 2)), "groupList dim only support 1 or 2(only when groupListType is 2)"),
     (dict(group_list_type=3), "groupListType"),
     (dict(act_type=3), "GELU_ERR_FUNC"),
     (dict(act_type=1), "actType 1"),

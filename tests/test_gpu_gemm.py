@@ -214,3 +214,59 @@ def test_register_kernel_epilogues(aclnn, oracle, dev, reg_path):
     torch.cuda.synchronize()
     assert np.abs(q.cpu().numpy().astype(np.int32) - q_ref.astype(np.int32)).max() <= 1
     np.testing.assert_allclose(qs.cpu().numpy(), s_ref, rtol=1e-2)
+
+
+# ------------------------------------------------------------------------------------------------ sparse group lists
+@pytest.mark.parametrize("M,K,N,E,order", [(300, 256, 256, 16, "ascending"), (640, 512, 520, 64, "ascending"),
+                                          (200, 128, 128, 8, "shuffled"), (96, 128, 72, 4, "all")])
+def test_sparse_group_list(aclnn, oracle, dev, M, K, N, E, order):
+    """groupListType 2: [E, 2] pairs (expert id, rows) in row order, ended by the first pair without rows
+    (gmm/grouped_matmul/op_kernel/grouped_matmul.h:288-345).  The oracle sees the same problem as a dense count list over
+    the weights picked by the pairs."""
+    rng = np.random.default_rng(M + E)
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
+    used = E if order == "all" else max(1, E // 3)
+    keys = np.sort(rng.choice(E, used, replace=False))
+    if order == "shuffled":
+        rng.shuffle(keys)
+    covered = M - 11                                              # the last rows belong to no pair
+    counts = rng.multinomial(covered - used, np.ones(used) / used) + 1
+    pairs = np.zeros((E, 2), np.int64)
+    pairs[:used, 0], pairs[:used, 1] = keys, counts
+    pairs[used:, 0] = rng.integers(0, E, E - used)                # ids behind the end marker are never read as groups
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    xd, wv = torch.from_numpy(x).to(dev), torch.from_numpy(wt).to(dev).transpose(1, 2)
+    out = torch.full((M, N), -7, dtype=torch.int32, device=dev)
+    aclnn.grouped_matmul_v4([xd], [wv], group_list=torch.from_numpy(pairs).to(dev), split_item=3, group_type=0,
+                            group_list_type=2, out=[out])
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    aclnn.grouped_matmul_v4([xd], [wv], scale=[torch.from_numpy(scale).to(dev)], per_token_scale=[torch.from_numpy(pt).to(dev)],
+                            group_list=torch.from_numpy(pairs).to(dev), split_item=3, group_type=0, group_list_type=2, out=[y])
+    torch.cuda.synchronize()
+    ref = oracle.grouped_matmul_i32(x, wt[keys], counts.astype(np.int64), list_type=1, w_trans=True)
+    got = out.cpu().numpy()
+    assert np.array_equal(got[:covered], ref[:covered])
+    assert (got[covered:] == -7).all()
+    ref_y = oracle.grouped_matmul_dequant(x, wt[keys], scale[keys], pt, counts.astype(np.int64), list_type=1, w_trans=True,
+                                          out_dtype=oracle.DT_BF16)
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16)[:covered], ref_y[:covered])
+
+
+def test_sparse_list_from_routing_v3(aclnn, oracle, dev):
+    """MoeInitRoutingV3's key/value count output is the sparse list GroupedMatmulV4 takes."""
+    rng = np.random.default_rng(3)
+    T, K, E, H, N = 96, 2, 32, 128, 64
+    x = rng.integers(-127, 128, (T, H)).astype(np.int8)
+    idx = rng.choice(E // 4, (T, K)).astype(np.int32) * 4          # only every fourth expert is used
+    wt = rng.integers(-127, 128, (E, N, H)).astype(np.int8)
+    ex, _, pairs, _ = aclnn.moe_init_routing_v3(torch.from_numpy(x).to(dev), torch.from_numpy(idx).to(dev), None,
+                                                expert_num=E, expert_tokens_num_type=2)
+    out = torch.zeros((T * K, N), dtype=torch.int32, device=dev)
+    aclnn.grouped_matmul_v4([ex], [torch.from_numpy(wt).to(dev).transpose(1, 2)], group_list=pairs, split_item=3,
+                            group_type=0, group_list_type=2, out=[out])
+    torch.cuda.synchronize()
+    ex_r, _, cnt_r, _ = oracle.moe_init_routing_v3(x, idx, None, E, None, 1, 1)
+    ref = oracle.grouped_matmul_i32(ex_r, wt, cnt_r, list_type=1, w_trans=True)
+    assert np.array_equal(out.cpu().numpy(), ref)
