@@ -99,3 +99,18 @@ class MoeFfnW8A8:
                                 out=[self.y], workspace=self.workspace)
         aclnn.moe_finalize_routing_v2(self.y, self.expanded_row_idx, scales=topk_weight, drop_pad_mode=2, out=self.out)
         return self.out
+
+    def capture(self, xq, x_scale, topk_idx, topk_weight):
+        """Records one pass over these input buffers into a HIP graph and returns (graph, out).
+
+        ``graph.replay()`` re-runs the recorded kernels on whatever the four input buffers hold at that time (same
+        shapes, same addresses) and leaves the result in ``out``.  The first phases (validation, planning) ran once,
+        at capture time: a replay is the second phases only, enqueued with a single launch.  One eager pass comes
+        first so that buffers, the workspace and kernel attributes exist before recording starts; nothing in the second
+        phases allocates, synchronises or clears memory with a memset node."""
+        self.forward(xq, x_scale, topk_idx, topk_weight)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = self.forward(xq, x_scale, topk_idx, topk_weight)
+        return graph, out

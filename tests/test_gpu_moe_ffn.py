@@ -89,3 +89,27 @@ def test_v2_and_v3_routing_chains_agree(pkg, dev):
         outs.append(ffn.forward(t(xq), t(xs), t(idx), t(wgt)).clone())
         torch.cuda.synchronize()
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
+def test_graph_replays_match_eager(pkg, dev):
+    """The pass recorded into a HIP graph: every replay, with eager work and synchronisations in between and new
+    contents in the input buffers, equals the eager pass on the same contents bit for bit."""
+    cfg = pkg.synth.config(0)
+    w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=0)
+    ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s)
+    eager = pkg.MoeFfnW8A8(w13, w13s, w2, w2s)
+    idx, wgt = pkg.synth.make_routing(cfg, seed=0)
+    xq, xs = pkg.synth.make_activations(cfg, seed=0)
+    bufs = [torch.from_numpy(a).to(dev) for a in (xq, xs, idx, wgt)]
+    graph, out = ffn.capture(*bufs)
+    for seed in (0, 1, 2, 1, 3):
+        idx, wgt = pkg.synth.make_routing(cfg, seed=seed)
+        xq, xs = pkg.synth.make_activations(cfg, seed=seed)
+        fresh = [torch.from_numpy(a).to(dev) for a in (xq, xs, idx, wgt)]
+        want = eager.forward(*fresh).clone()          # eager work between the replays
+        torch.cuda.synchronize()
+        for dst, src in zip(bufs, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16)), seed
