@@ -15,9 +15,13 @@
  * sharedInput BF16 or FLOAT16 [rows, n] with sharedInputOffset + rows <= batch; dtype must be 0 (FLOAT);
  * transposeX1 / transposeX2 false; groupListType 0 (cumsum) or 1 (count).
  *
- * This build takes x2 as INT8 [e, k, n] (ND; the K-contiguous storage seen through a transposed view is the fast
- * layout, as for aclnnGroupedMatmulV4).  The reference's ND entry points take only INT4 weights packed in INT32 (its INT8
- * weights go through the FRACTAL_NZ entry points); those are rejected here with ACLNN_ERR_PARAM_INVALID.  bias,
+ * aclnnGroupedMatmulFinalizeRoutingWeightNz / WeightNzV2 (replacing aclnn_grouped_matmul_finalize_routing_weight_nz.h:48-53
+ * and aclnn_grouped_matmul_finalize_routing_weight_nz_v2.h:55-61) are the reference's route for INT8 weights: x2 is stored
+ * in the blocked FRACTAL_NZ layout [e, n/32, k/16, 16, 32] (storage shape; the view shape is that or [e, k, n]).
+ *
+ * This build also takes x2 as INT8 [e, k, n] ND in the plain entry points (the K-contiguous storage seen through a
+ * transposed view is the fast ND layout, as for aclnnGroupedMatmulV4).  The reference's ND entry points take only INT4
+ * weights packed in INT32; those are rejected here with ACLNN_ERR_PARAM_INVALID.  bias,
  * pertokenScale, sharedInput and logit may be null (no bias / scale 1 / no shared rows / weight 1); offset and the
  * antiquant arguments must be null.
  */
@@ -58,6 +62,24 @@ ACLNN_API aclnnStatus aclnnGroupedMatmulFinalizeRoutingV3GetWorkspaceSize(
     const aclIntArray* tuningConfigOptional, aclTensor* out, uint64_t* workspaceSize, aclOpExecutor** executor);
 ACLNN_API aclnnStatus aclnnGroupedMatmulFinalizeRoutingV3(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
                                                           aclrtStream stream);
+
+ACLNN_API aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNzGetWorkspaceSize(
+    const aclTensor* x1, const aclTensor* x2, const aclTensor* scale, const aclTensor* bias,
+    const aclTensor* pertokenScaleOptional, const aclTensor* groupList, const aclTensor* sharedInput, const aclTensor* logit,
+    const aclTensor* rowIndex, int64_t dtype, float sharedInputWeight, int64_t sharedInputOffset, bool transposeX1,
+    bool transposeX2, int64_t groupListType, aclTensor* out, uint64_t* workspaceSize, aclOpExecutor** executor);
+ACLNN_API aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNz(void* workspace, uint64_t workspaceSize,
+                                                                aclOpExecutor* executor, aclrtStream stream);
+
+ACLNN_API aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNzV2GetWorkspaceSize(
+    const aclTensor* x1, aclTensor* x2, const aclTensor* scale, const aclTensor* bias, const aclTensor* offsetOptional,
+    const aclTensor* antiquantScaleOptional, const aclTensor* antiquantOffsetOptional,
+    const aclTensor* pertokenScaleOptional, const aclTensor* groupList, const aclTensor* sharedInput, const aclTensor* logit,
+    const aclTensor* rowIndex, int64_t dtype, float sharedInputWeight, int64_t sharedInputOffset, bool transposeX1,
+    bool transposeX2, int64_t groupListType, const aclIntArray* tuningConfigOptional, aclTensor* out,
+    uint64_t* workspaceSize, aclOpExecutor** executor);
+ACLNN_API aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNzV2(void* workspace, uint64_t workspaceSize,
+                                                                  aclOpExecutor* executor, aclrtStream stream);
 
 #ifdef __cplusplus
 }

@@ -16,6 +16,7 @@ _LIB_PATH = os.environ.get("OPAPI_LIBRARY_PATH") or os.path.join(_HERE, "lib", "
 
 ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32, ACL_INT64, ACL_BOOL, ACL_BF16 = 0, 1, 2, 3, 9, 12, 27
 ACL_FORMAT_ND = 2
+ACL_FORMAT_FRACTAL_NZ = 29
 
 ACLNN_SUCCESS = 0
 ACLNN_ERR_PARAM_NULLPTR = 161001
@@ -61,20 +62,29 @@ _PHASE1_SIGNATURES = {
         [_VP, _VP, _VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _I64, _VP, _I64, _VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulSwigluQuantWeightNZGetWorkspaceSize":
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulV4GetWorkspaceSize":
         [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulV5GetWorkspaceSize":
         [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulWeightNzGetWorkspaceSize":
+        [_VP] * 12 + [_I64, _I64, _I64, _I64] + [_VP, _I64, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulFinalizeRoutingV3GetWorkspaceSize":
         [_VP] * 12 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulFinalizeRoutingV2GetWorkspaceSize":
         [_VP] * 12 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _U64P, _VPP],
     "aclnnGroupedMatmulFinalizeRoutingGetWorkspaceSize":
         [_VP] * 9 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulFinalizeRoutingWeightNzGetWorkspaceSize":
+        [_VP] * 9 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _U64P, _VPP],
+    "aclnnGroupedMatmulFinalizeRoutingWeightNzV2GetWorkspaceSize":
+        [_VP] * 12 + [_I64, ctypes.c_float, _I64, ctypes.c_bool, ctypes.c_bool, _I64, _VP, _VP, _U64P, _VPP],
     "aclnnMoeFinalizeRoutingV2GetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _U64P, _VPP],
 }
-_PHASE2 = ["aclnnGroupedMatmulFinalizeRouting", "aclnnGroupedMatmulFinalizeRoutingV2", "aclnnGroupedMatmulFinalizeRoutingV3",
+_PHASE2 = ["aclnnGroupedMatmulSwigluQuantWeightNZ", "aclnnGroupedMatmulWeightNz",
+           "aclnnGroupedMatmulFinalizeRoutingWeightNz", "aclnnGroupedMatmulFinalizeRoutingWeightNzV2", "aclnnGroupedMatmulFinalizeRouting", "aclnnGroupedMatmulFinalizeRoutingV2", "aclnnGroupedMatmulFinalizeRoutingV3",
            "aclnnMoeGatingTopKSoftmaxV2", "aclnnMoeInitRoutingV2", "aclnnMoeInitRoutingV3", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
            "aclnnMoeFinalizeRoutingV2"]
 
@@ -117,16 +127,18 @@ def last_error():
 
 
 # ------------------------------------------------------------------------------------------------ descriptors
-def create_tensor(shape, dtype_code, data_ptr, strides=None, offset=0, fmt=ACL_FORMAT_ND):
+def create_tensor(shape, dtype_code, data_ptr, strides=None, offset=0, fmt=ACL_FORMAT_ND, storage_shape=None):
     """Raw aclCreateTensor; the caller destroys the handle (or hands it to a tensor list)."""
     n = len(shape)
     dims = (_I64 * max(n, 1))(*shape)
+    storage = list(shape) if storage_shape is None else list(storage_shape)
+    sdims = (_I64 * max(len(storage), 1))(*storage)
     if strides is None:
         strides = [1] * n
         for i in range(n - 2, -1, -1):
             strides[i] = strides[i + 1] * shape[i + 1]
     st = (_I64 * max(n, 1))(*strides)
-    h = lib().aclCreateTensor(dims, n, dtype_code, st, offset, fmt, dims, n, _VP(data_ptr))
+    h = lib().aclCreateTensor(dims, n, dtype_code, st, offset, fmt, sdims, len(storage), _VP(data_ptr))
     if not h:
         raise MemoryError("aclCreateTensor failed")
     return h
@@ -153,6 +165,11 @@ class _Handles:
         h = tensor_of(t)
         self.tensors.append(h)
         return h
+
+    def raw(self, handle):
+        """Takes ownership of a handle made with create_tensor."""
+        self.tensors.append(handle)
+        return handle
 
     def tensor_list(self, ts):
         if ts is None:
@@ -315,12 +332,24 @@ def moe_init_routing_v3(x, expert_idx, scale=None, expert_num=0, expert_tokens_n
     return expanded_x, row_idx, counts, expanded_scale
 
 
+def nz_weight_handle(weight_nz, view_3d=False, fmt=ACL_FORMAT_FRACTAL_NZ):
+    """Descriptor of a blocked weight held as a contiguous torch tensor [E, N/32, K/16, 16, 32].  view_3d: describe it
+    through the 3-D view [E, K, N] over that storage (the form aclnn...WeightNZ entry points accept as well)."""
+    E, n1, k1, k0, n0 = weight_nz.shape
+    assert (k0, n0) == (16, 32) and weight_nz.is_contiguous()
+    shape = [E, k1 * 16, n1 * 32] if view_3d else list(weight_nz.shape)
+    return create_tensor(shape, _DTYPE_CODE[weight_nz.dtype], weight_nz.data_ptr(), None, 0, fmt, list(weight_nz.shape))
+
+
 def grouped_matmul_swiglu_quant(x, weight, group_list, weight_scale, x_scale, bias=None, offset=None, out=None,
-                                workspace=None):
+                                workspace=None, weight_nz=None):
     """aclnnGroupedMatmulSwigluQuant.  weight is the [E, K, N] view (contiguous, or ``storage.transpose(1, 2)`` over
-    [E, N, K] storage).  Returns (output int8 [M, N/2], output_scale fp32 [M])."""
+    [E, N, K] storage); or pass weight=None and weight_nz=(tensor [E, N/32, K/16, 16, 32], how) with how one of
+    "nz5d" (FRACTAL_NZ 5-D tensor through the plain entry point), "entry5d" / "entry3d" (through
+    aclnnGroupedMatmulSwigluQuantWeightNZ, 5-D shape or 3-D view, ND format field).
+    Returns (output int8 [M, N/2], output_scale fp32 [M])."""
     M = x.shape[0]
-    N = weight.shape[2]
+    N = weight.shape[2] if weight is not None else weight_nz[0].shape[1] * 32
     dev = x.device
     if out is not None:
         output, output_scale = out
@@ -329,9 +358,19 @@ def grouped_matmul_swiglu_quant(x, weight, group_list, weight_scale, x_scale, bi
         output_scale = torch.empty((M,), dtype=torch.float32, device=dev)
     h = _Handles()
     try:
-        args = [h.tensor(x), h.tensor(weight), h.tensor(bias), h.tensor(offset), h.tensor(weight_scale),
+        api = "aclnnGroupedMatmulSwigluQuant"
+        if weight is not None:
+            wh = h.tensor(weight)
+        else:
+            tensor, how = weight_nz
+            if how == "nz5d":
+                wh = h.raw(nz_weight_handle(tensor))
+            else:
+                api = "aclnnGroupedMatmulSwigluQuantWeightNZ"
+                wh = h.raw(nz_weight_handle(tensor, view_3d=(how == "entry3d"), fmt=ACL_FORMAT_ND))
+        args = [h.tensor(x), wh, h.tensor(bias), h.tensor(offset), h.tensor(weight_scale),
                 h.tensor(x_scale), h.tensor(group_list), h.tensor(output), h.tensor(output_scale), None]
-        _run_two_phase("aclnnGroupedMatmulSwigluQuant", args, dev, workspace)
+        _run_two_phase(api, args, dev, workspace)
     finally:
         h.close()
     return output, output_scale
@@ -340,28 +379,44 @@ def grouped_matmul_swiglu_quant(x, weight, group_list, weight_scale, x_scale, bi
 def grouped_matmul_v4(x, weight, bias=None, scale=None, offset=None, antiquant_scale=None, antiquant_offset=None,
                       per_token_scale=None, group_list=None, activation_input=None, activation_quant_scale=None,
                       activation_quant_offset=None, split_item=0, group_type=-1, group_list_type=0, act_type=0,
-                      output_dtype=None, out=None, workspace=None, tuning_config=None):
+                      output_dtype=None, out=None, workspace=None, tuning_config=None, weight_nz=None):
     """aclnnGroupedMatmulV4, or aclnnGroupedMatmulV5 when tuning_config (a list of ints whose first value is the expected
     number of rows per expert) is given.  x / weight / scale / per_token_scale / out are lists of tensors as in the
-    reference.  Returns the list of outputs."""
+    reference.  weight_nz=(tensor [E, N/32, K/16, 16, 32], how) instead of weight passes a blocked weight: how "nz5d"
+    (FRACTAL_NZ 5-D tensor through V4 / V5) or "entry5d" / "entry3d" (aclnnGroupedMatmulWeightNz, 5-D shape or 3-D view).
+    Returns the list of outputs."""
     dev = x[0].device
+    n_out = weight[0].shape[2] if weight is not None else weight_nz[0].shape[1] * 32
     if out is None:
         if output_dtype is None:
             output_dtype = torch.int32 if scale is None else (
                 torch.bfloat16 if scale[0].dtype == torch.bfloat16 else torch.float16)
-        out = [torch.empty((x[0].shape[0], weight[0].shape[2]), dtype=output_dtype, device=dev)]
+        out = [torch.empty((x[0].shape[0], n_out), dtype=output_dtype, device=dev)]
     h = _Handles()
     try:
-        args = [h.tensor_list(x), h.tensor_list(weight), h.tensor_list(bias), h.tensor_list(scale),
+        api = "aclnnGroupedMatmulV5" if tuning_config is not None else "aclnnGroupedMatmulV4"
+        if weight is not None:
+            wl = h.tensor_list(weight)
+        else:
+            tensor, how = weight_nz
+            if how == "nz5d":
+                wh = nz_weight_handle(tensor)
+            else:
+                api = "aclnnGroupedMatmulWeightNz"
+                wh = nz_weight_handle(tensor, view_3d=(how == "entry3d"), fmt=ACL_FORMAT_ND)
+            wl = lib().aclCreateTensorList((_VP * 1)(wh), 1)
+            h.lists.append(wl)
+        args = [h.tensor_list(x), wl, h.tensor_list(bias), h.tensor_list(scale),
                 h.tensor_list(offset), h.tensor_list(antiquant_scale), h.tensor_list(antiquant_offset),
                 h.tensor_list(per_token_scale), h.tensor(group_list), h.tensor_list(activation_input),
                 h.tensor_list(activation_quant_scale), h.tensor_list(activation_quant_offset), split_item, group_type,
                 group_list_type, act_type]
-        if tuning_config is not None:
+        if api == "aclnnGroupedMatmulWeightNz":
+            args += [h.int_array(tuning_config), 0]          # tuningConfigOptional (may be null), quantGroupSize
+        elif tuning_config is not None:
             args.append(h.int_array(tuning_config))
         args += [h.tensor_list(out), None, None]
-        _run_two_phase("aclnnGroupedMatmulV5" if tuning_config is not None else "aclnnGroupedMatmulV4", args, dev,
-                       workspace)
+        _run_two_phase(api, args, dev, workspace)
     finally:
         h.close()
     return out
@@ -374,19 +429,29 @@ def grouped_matmul_v5(x, weight, tuning_config=(), **kwargs):
 
 def grouped_matmul_finalize_routing(x, weight, scale, row_index, batch, group_list, group_list_type=1, bias=None,
                                     per_token_scale=None, logit=None, shared_input=None, shared_input_weight=1.0,
-                                    shared_input_offset=0, tuning_config=None, out=None, workspace=None, version=3):
+                                    shared_input_offset=0, tuning_config=None, out=None, workspace=None, version=3,
+                                    weight_nz=None):
     """aclnnGroupedMatmulFinalizeRouting (version 1), V2 or V3: int8 grouped matmul fused with the weighted combine.
-    weight is the [E, K, N] view; returns out fp32 [batch, N]."""
+    weight is the [E, K, N] view; or weight=None and weight_nz = blocked tensor [E, N/32, K/16, 16, 32], which goes
+    through aclnnGroupedMatmulFinalizeRoutingWeightNz (version 1) or WeightNzV2 (any other version) as a 3-D view.
+    Returns out fp32 [batch, N]."""
     dev = x.device
-    N = weight.shape[2]
+    N = weight.shape[2] if weight is not None else weight_nz.shape[1] * 32
     if out is None:
         out = torch.empty((batch, N), dtype=torch.float32, device=dev)
     h = _Handles()
     try:
-        head = [h.tensor(x), h.tensor(weight), h.tensor(scale), h.tensor(bias)]
+        wh = h.tensor(weight) if weight is not None else h.raw(nz_weight_handle(weight_nz, view_3d=True, fmt=ACL_FORMAT_ND))
+        head = [h.tensor(x), wh, h.tensor(scale), h.tensor(bias)]
         tail = [h.tensor(per_token_scale), h.tensor(group_list), h.tensor(shared_input), h.tensor(logit), h.tensor(row_index),
                 0, float(shared_input_weight), int(shared_input_offset), False, False, int(group_list_type)]
-        if version == 1:
+        if weight is None and version == 1:
+            api, args = "aclnnGroupedMatmulFinalizeRoutingWeightNz", head + tail + [h.tensor(out)]
+        elif weight is None:
+            api = "aclnnGroupedMatmulFinalizeRoutingWeightNzV2"
+            args = head + [None, None, None] + tail + [None if tuning_config is None else h.int_array(list(tuning_config)),
+                                                         h.tensor(out)]
+        elif version == 1:
             api, args = "aclnnGroupedMatmulFinalizeRouting", head + tail + [h.tensor(out)]
         elif version == 2:
             api, args = "aclnnGroupedMatmulFinalizeRoutingV2", head + [None, None, None] + tail + [h.tensor(out)]

@@ -22,6 +22,10 @@ struct Problem {
     const int8_t* x = nullptr;       // [M, K] row-major
     const int8_t* w = nullptr;       // per group: [N, K] K-contiguous when wKMajor, else [K, N] N-contiguous
     bool wKMajor = true;
+    // Blocked weight layout (the reference's FRACTAL_NZ for int8): per group [N/32][K/16][16][32], i.e. element (k, n)
+    // at ((n / 32) * (K / 16) + k / 16) * 512 + (k % 16) * 32 + n % 32.  Needs K % 16 == 0 and N % 32 == 0; wKMajor is
+    // then ignored.
+    bool wNz = false;
     int64_t M = 0, K = 0, N = 0;
     int32_t groups = 0;
     const void* groupList = nullptr; // device, int64 or int32: cumsum or counts [groups], or sparse pairs [groups, 2]

@@ -37,6 +37,8 @@
 namespace gemm {
 namespace {
 
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) v2i* LdsV2iPtr;
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float Float2 __attribute__((ext_vector_type(2)));
@@ -187,6 +189,7 @@ struct KernelArgs {
     int64_t wGroupStride;  // bytes between experts
     int64_t wStrideN;      // bytes between consecutive output channels
     int64_t wStrideK;      // bytes between consecutive k
+    int32_t wNz;           // weights in 32-channel x 16-k blocks ([N/32][K/16][16][32] per expert), see Problem::wNz
     int32_t M, K, N;
     int32_t groups;
     int32_t tilesN;
@@ -260,6 +263,12 @@ __device__ __forceinline__ float LoadScale(const void* p, int64_t i, int dtype) 
     const uint16_t raw = static_cast<const uint16_t*>(p)[i];
     if (dtype == 1) return __half2float(__ushort_as_half(raw));
     return __uint_as_float(static_cast<uint32_t>(raw) << 16);
+}
+
+// Byte offset of (channel n, k = 0) inside one expert's weights; consecutive k are a.wStrideK bytes apart (32 in the
+// blocked layout: a 32-channel block holds its K rows of 32 channel bytes back to back).
+__device__ __forceinline__ int64_t WeightRowBase(const KernelArgs& a, int32_t n) {
+    return a.wNz ? static_cast<int64_t>(n >> 5) * a.K * 32 + (n & 31) : static_cast<int64_t>(n) * a.wStrideN;
 }
 
 // Epilogue of one tile.  acc[mi][ni][v] is C[row, col] with row = waveRow0 + 32*mi + 8*(v/4) + 4*lhi + (v%4); the wave
@@ -569,9 +578,16 @@ __device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leavi
 
 // Persistent: the grid is one workgroup per CU (a multiple of 8); workgroup b serves XCD b % 8 and walks that XCD's
 // share of the tile list with stride gridDim / 8.
-template <int kSub0, int kSub1, int kStep, Epilogue kEpi>
+//
+// kNz: the weights come in the 32-channel x 16-k blocked layout.  A 32-channel block is then one contiguous stream of
+// K x 32 bytes, so a stage's weight part is eight 4 KB pieces that land in LDS as [block][k][32 channels]; the MFMA
+// operand (16 consecutive k of one channel per lane) is read back with the transposing LDS load ds_read_b64_tr_b8:
+// per 16 lanes, lanes 2r and 2r + 1 supply the two 8-byte halves of row r (r = 0..7) and lane i receives column i,
+// i.e. with rows = 8 consecutive k and columns = 16 channels each lane gets 8 consecutive k of its channel.
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz>
 __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     KernelArgs a, const int32_t* __restrict__ sched) {
+    static_assert(!kNz || kStep == 128, "the blocked weight layout is built for 128-byte k-steps");
     using Cfg = StreamCfg<kSub0, kSub1, kStep>;
     constexpr int kSubM = kSub0;  // accumulator tiles per wave (wave row 1 uses the first kSub1 of them)
     constexpr int kTileM = Cfg::kTileM;
@@ -629,6 +645,12 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                 const int c = (LdsOffset<kStep>(r, slot) >> 4) % Cfg::kChunksPerRow;
                 const bool wholeInstrPast = Cfg::kRowsPerInstr * j >= iss.rows;
                 laneOff[q] = wholeInstrPast ? 0u : static_cast<uint32_t>(min(r, iss.rows - 1) * a.K + c * kChunk);
+            } else if (kNz) {
+                // weight instruction jw moves 32 k-rows (x 32 channel bytes) of channel block jw / 4: 1 KB, contiguous
+                // in memory and in LDS; lane -> (k-row lane / 2, 16-byte half lane % 2)
+                const int jw = j - Cfg::kInstrA;
+                const int32_t block = ChannelOfRow<kSwiglu>(a, iss, 32 * (jw / 4)) >> 5;
+                laneOff[q] = static_cast<uint32_t>(block * a.K * 32 + ((jw % 4) * 32 + lane / 2) * 32 + (lane % 2) * kChunk);
             } else {
                 const int r = Cfg::kRowsPerInstr * (j - Cfg::kInstrA) + rowIn;
                 const int c = (LdsOffset<kStep>(r, slot) >> 4) % Cfg::kChunksPerRow;
@@ -639,10 +661,11 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     auto issueStage = [&](int ring) {
         const uint32_t dst = ldsBase + ring * kStageBytes;
         const int kOff = issStep * kStep;
+        const int kOffW = kNz ? kOff * 32 : kOff;  // blocked layout: one k is 32 bytes further
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
             const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
-            DmaToLdsAddr16((j < Cfg::kInstrA ? issX : issW) + kOff, laneOff[q], dst + j * 1024);
+            DmaToLdsAddr16(j < Cfg::kInstrA ? issX + kOff : issW + kOffW, laneOff[q], dst + j * 1024);
         }
         if (++issStep == kSteps) {
             // move to this workgroup's next tile; past the last one the same tile is fetched again into ring slots
@@ -703,8 +726,24 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             auto loadSlice = [&](int ks, int buf) {
                 if (kMy == 0) return;
                 const int chunk = 2 * ks + lhi;
-                bf[buf][0] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + l32, chunk));
-                bf[buf][1] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + bRowStep + l32, chunk));
+                if constexpr (kNz) {
+                    // 16-lane group g: channels 16 * (g % 2) .. + 15 of the block, k-half g / 2 (= lhi) of the slice;
+                    // lane j of the group supplies bytes (k = kBase + j / 2, channels 8 * (j % 2) .. + 7)
+                    const int j = lane & 15;
+                    const int inBlock = (32 * ks + 16 * lhi + (j >> 1)) * 32 + 16 * ((lane >> 4) & 1) + 8 * (j & 1);
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni) {
+                        // addressed through the 32-bit LDS address: no generic-to-LDS pointer conversion in the loop
+                        const uint32_t blk = ldsBase + ring * kStageBytes + kTileM * kStep +
+                                             ((bRow0 + ni * bRowStep) >> 5) * 4096 + inBlock;
+                        const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk));
+                        const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk + 8 * 32));
+                        bf[buf][ni] = v4i{lo[0], lo[1], hi[0], hi[1]};
+                    }
+                } else {
+                    bf[buf][0] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + l32, chunk));
+                    bf[buf][1] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + bRowStep + l32, chunk));
+                }
 #pragma unroll
                 for (int mi = 0; mi < kMy; ++mi) {
                     af[buf][mi] = *reinterpret_cast<const v4i*>(A + LdsOffset<kStep>(waveRow0 + mi * 32 + l32, chunk));
@@ -1214,7 +1253,7 @@ __global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a, const int
             const int p = i * kThreads + tid;
             const int r = p % kTileN;
             const int chunk = p / kTileN;
-            const int8_t* src = wGroup + static_cast<int64_t>(ChannelOfRow<kSwiglu>(a, t, r)) * a.wStrideN;
+            const int8_t* src = wGroup + WeightRowBase(a, ChannelOfRow<kSwiglu>(a, t, r));
             union { v4i v; int8_t b[16]; } u;
             for (int j = 0; j < kChunk; ++j) {
                 const int k = k0 + chunk * kChunk + j;
@@ -1303,10 +1342,10 @@ int DeviceCuCount() {
     return count;
 }
 
-template <int kSub0, int kSub1, int kStep, Epilogue kEpi>
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz>
 hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
     using Cfg = StreamCfg<kSub0, kSub1, kStep>;
-    auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi>;
+    auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi, kNz>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
     if (attr != hipSuccess) return attr;
@@ -1321,17 +1360,23 @@ hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t ma
 
 // Tile heights and their (wave row 0, wave row 1, k-step) shapes.  128-byte steps with a ring of three or more stages
 // stream best; 192 and 256 rows only leave room for two such stages.
+template <Epilogue kEpi, bool kNz>
+hipError_t LaunchStreamShapeOf(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
+    switch (plan.tileM) {
+        case 32: return LaunchStream<1, 0, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+        case 64: return LaunchStream<1, 1, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+        case 96: return LaunchStream<2, 1, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+        case 128: return LaunchStream<2, 2, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+        case 160: return LaunchStream<3, 2, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+        case 192: return LaunchStream<3, 3, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+        default: return LaunchStream<4, 4, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+    }
+}
+
 template <Epilogue kEpi>
 hipError_t LaunchStreamShape(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
-    switch (plan.tileM) {
-        case 32: return LaunchStream<1, 0, 128, kEpi>(args, sched, plan.maxTiles, stream);
-        case 64: return LaunchStream<1, 1, 128, kEpi>(args, sched, plan.maxTiles, stream);
-        case 96: return LaunchStream<2, 1, 128, kEpi>(args, sched, plan.maxTiles, stream);
-        case 128: return LaunchStream<2, 2, 128, kEpi>(args, sched, plan.maxTiles, stream);
-        case 160: return LaunchStream<3, 2, 128, kEpi>(args, sched, plan.maxTiles, stream);
-        case 192: return LaunchStream<3, 3, 128, kEpi>(args, sched, plan.maxTiles, stream);
-        default: return LaunchStream<4, 4, 128, kEpi>(args, sched, plan.maxTiles, stream);
-    }
+    return args.wNz ? LaunchStreamShapeOf<kEpi, true>(plan, args, sched, stream)
+                    : LaunchStreamShapeOf<kEpi, false>(plan, args, sched, stream);
 }
 
 template <int kSubM, void (*kKernel)(KernelArgs, const int32_t*)>
@@ -1386,7 +1431,8 @@ hipError_t LaunchGenericShape(const Plan& plan, const KernelArgs& args, const in
 // The DMA ring needs K-contiguous weights, whole 128-byte k steps, 16-byte aligned bases and 32-bit offsets inside one
 // expert's weights.
 bool StreamOk(const Problem& p) {
-    return p.wKMajor && p.K % 128 == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
+    const bool layoutOk = p.wNz ? (p.N % 32 == 0 && (p.epilogue != Epilogue::kSwiglu || (p.N / 2) % 32 == 0)) : p.wKMajor;
+    return layoutOk && p.K % 128 == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
            reinterpret_cast<uintptr_t>(p.w) % kChunk == 0 && p.N * p.K < (1ll << 31);
 }
 
@@ -1421,7 +1467,7 @@ Plan MakePlan(const Problem& p) {
     {
         // read at plan time (not cached) so that one process can plan either way
         const char* env = std::getenv("OPAPI_GEMM_PATH");
-        plan.regPath = StreamOk(p) && plan.tileM <= 192 && p.combineIndex == nullptr && env != nullptr &&
+        plan.regPath = StreamOk(p) && !p.wNz && plan.tileM <= 192 && p.combineIndex == nullptr && env != nullptr &&
                        std::string(env) == "reg";
     }
     plan.wavesM = plan.tileM >= 64 && StreamOk(p) ? 2 : 1;
@@ -1474,7 +1520,8 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.w = p.w;
     ka.wGroupStride = p.K * p.N;
     ka.wStrideN = p.wKMajor ? p.K : 1;
-    ka.wStrideK = p.wKMajor ? 1 : p.N;
+    ka.wStrideK = p.wNz ? 32 : (p.wKMajor ? 1 : p.N);
+    ka.wNz = p.wNz ? 1 : 0;
     ka.M = static_cast<int32_t>(p.M);
     ka.K = static_cast<int32_t>(p.K);
     ka.N = static_cast<int32_t>(p.N);

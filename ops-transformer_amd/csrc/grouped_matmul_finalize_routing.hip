@@ -104,7 +104,7 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
                         const aclTensor* antiquantOffset, const aclTensor* perToken, const aclTensor* groupList,
                         const aclTensor* sharedInput, const aclTensor* logit, const aclTensor* rowIndex, int64_t dtype,
                         float sharedInputWeight, int64_t sharedInputOffset, bool transposeX1, bool transposeX2,
-                        int64_t groupListType, const aclIntArray* tuningConfig, const aclTensor* out,
+                        int64_t groupListType, const aclIntArray* tuningConfig, bool forceNz, const aclTensor* out,
                         uint64_t* workspaceSize, aclOpExecutor** executor) {
     using namespace opapi;
     ClearError();
@@ -124,7 +124,15 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
     OPAPI_CHECK(x2->dtype != ACL_INT32 && x2->dtype != ACL_INT4, kInvalid,
                 "INT4 weights (packed in INT32) are not built here: this build's fused combine takes INT8 weights");
     OPAPI_CHECK(x2->dtype == ACL_INT8, kInvalid, "x1 and x2 dtype should be same (INT8), actual x2 dtype is %d.", (int)x2->dtype);
-    OPAPI_CHECK(x2->format == ACL_FORMAT_ND, kInvalid, "x2's format should be ND (FRACTAL_NZ weights are not built here).");
+    // a blocked (FRACTAL_NZ) INT8 weight: [E, N/32, K/16, 16, 32] as a 5-D tensor or as the 3-D view [E, K, N] over
+    // storage of that shape; the WeightNz entry points take the storage shape as the only evidence
+    const bool nz = forceNz || x2->format == ACL_FORMAT_FRACTAL_NZ;
+    OPAPI_CHECK(nz || x2->format == ACL_FORMAT_ND, kInvalid, "x2's format should be ND or FRACTAL_NZ. actual is [%d].",
+                (int)x2->format);
+    const std::vector<int64_t>& blocked = x2->dims.size() == 5 ? x2->dims : x2->storage;
+    OPAPI_CHECK(!nz || ((x2->dims.size() == 5 || x2->dims.size() == 3) && blocked.size() == 5 && blocked[3] == 16 &&
+                        blocked[4] == 32), kInvalid,
+                "x2'format only support NZ, but now x2's format is not NZ: the storage shape must be [E, N/32, K/16, 16, 32].");
     OPAPI_CHECK(offset == nullptr, kInvalid, "offset belongs to the INT4 case and must be nullptr with INT8 weights");
     OPAPI_CHECK(scale->dtype == ACL_FLOAT || scale->dtype == ACL_BF16, kInvalid, "scale must be FLOAT or BF16");
     OPAPI_CHECK(bias == nullptr || bias->dtype == ACL_BF16 || bias->dtype == ACL_FLOAT, kInvalid, "bias must be BF16 or FLOAT");
@@ -138,11 +146,16 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
 
     // ranks and extents
     OPAPI_CHECK(x1->dims.size() == 2, kInvalid, "input x Dims is %zu, weight Dims is %zu.", x1->dims.size(), x2->dims.size());
-    OPAPI_CHECK(x2->dims.size() == 3, kInvalid, "input x Dims is %zu, weight Dims is %zu.", x1->dims.size(), x2->dims.size());
+    OPAPI_CHECK(x2->dims.size() == 3 || (nz && x2->dims.size() == 5), kInvalid, "input x Dims is %zu, weight Dims is %zu.",
+                x1->dims.size(), x2->dims.size());
     OPAPI_CHECK(out->dims.size() == 2, kInvalid, "Out dim num should be equal to 2, but is %zu.", out->dims.size());
-    const int64_t m = x1->dims[0], k = x1->dims[1], e = x2->dims[0], n = x2->dims[2], batch = out->dims[0];
-    OPAPI_CHECK(x2->dims[1] == k, kInvalid, "x1 k dim and x2 k dim should be same, but are %lld and %lld.", (long long)k,
-                (long long)x2->dims[1]);
+    const int64_t m = x1->dims[0], k = x1->dims[1], e = x2->dims[0], batch = out->dims[0];
+    const int64_t n = x2->dims.size() == 5 ? x2->dims[1] * 32 : x2->dims[2];
+    const int64_t wk = x2->dims.size() == 5 ? x2->dims[2] * 16 : x2->dims[1];
+    OPAPI_CHECK(wk == k, kInvalid, "x1 k dim and x2 k dim should be same, but are %lld and %lld.", (long long)k, (long long)wk);
+    OPAPI_CHECK(!nz || (blocked[0] == e && blocked[1] * 32 == n && blocked[2] * 16 == k && x2->offset == 0), kInvalid,
+                "the blocked weight storage must be [%lld, %lld, %lld, 16, 32] (N a multiple of 32, K of 16)", (long long)e,
+                (long long)(n / 32), (long long)(k / 16));
     const bool scale2d = scale->dims.size() == 2 && scale->dims[0] == e && scale->dims[1] == n;
     const bool scale3d = scale->dims.size() == 3 && scale->dims[0] == e && scale->dims[1] == 1 && scale->dims[2] == n;
     OPAPI_CHECK(scale->dims.empty() || scale->dims[0] == e, kInvalid,
@@ -191,8 +204,8 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
                     (long long)expected);
     }
 
-    const bool wTransposed = IsLastTwoDimsTransposed(x2);
-    OPAPI_CHECK(wTransposed || IsContiguous(x2), kInvalid,
+    const bool wTransposed = !nz && IsLastTwoDimsTransposed(x2);
+    OPAPI_CHECK(nz || wTransposed || IsContiguous(x2), kInvalid,
                 "x2 must be contiguous [E,K,N] or the transposed view of contiguous [E,N,K] storage");
     const aclTensor* plain[] = {x1, scale, bias, perToken, groupList, sharedInput, logit, rowIndex, out};
     for (const aclTensor* t : plain) {
@@ -220,6 +233,7 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
     p.x = reinterpret_cast<const int8_t*>(DataPtr(x1));
     p.w = reinterpret_cast<const int8_t*>(DataPtr(x2));
     p.wKMajor = wTransposed;
+    p.wNz = nz;
     p.M = batch == 0 ? 0 : m;
     p.K = k;
     p.N = n;
@@ -264,8 +278,8 @@ extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingGetWorkspaceSize(
     uint64_t* workspaceSize, aclOpExecutor** executor) {
     return PlanCombine("GroupedMatmulFinalizeRouting weightNd", x, w, scaleOptional, biasOptional, nullptr, nullptr, nullptr,
                        pertokenScaleOptional, groupListOptional, sharedInputOptional, logitOptional, rowIndexOptional, dtype,
-                       sharedInputWeight, sharedInputOffset, transposeX, transposeW, groupListType, nullptr, y, workspaceSize,
-                       executor);
+                       sharedInputWeight, sharedInputOffset, transposeX, transposeW, groupListType, nullptr, /*forceNz=*/false, y,
+                       workspaceSize, executor);
 }
 
 extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRouting(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
@@ -283,7 +297,7 @@ extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingV2GetWorkspaceSize(
     return PlanCombine("GroupedMatmulFinalizeRoutingV2 weightNd", x1, x2, scaleOptional, biasOptional, offsetOptional,
                        antiquantScaleOptional, antiquantOffsetOptional, pertokenScaleOptional, groupListOptional,
                        sharedInputOptional, logitOptional, rowIndexOptional, dtype, sharedInputWeight, sharedInputOffset,
-                       transposeX1, transposeX2, groupListType, nullptr, out, workspaceSize, executor);
+                       transposeX1, transposeX2, groupListType, nullptr, /*forceNz=*/false, out, workspaceSize, executor);
 }
 
 extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
@@ -301,10 +315,46 @@ extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingV3GetWorkspaceSize(
     return PlanCombine("aclnnGroupedMatmulFinalizeRoutingV3 weightNd", x1, x2, scaleOptional, biasOptional, offsetOptional,
                        antiquantScaleOptional, antiquantOffsetOptional, pertokenScaleOptional, groupListOptional,
                        sharedInputOptional, logitOptional, rowIndexOptional, dtype, sharedInputWeight, sharedInputOffset,
-                       transposeX1, transposeX2, groupListType, tuningConfigOptional, out, workspaceSize, executor);
+                       transposeX1, transposeX2, groupListType, tuningConfigOptional, /*forceNz=*/false, out, workspaceSize,
+                       executor);
 }
 
 extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingV3(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
                                                            aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
+}
+
+// The FRACTAL_NZ entry points (aclnn_grouped_matmul_finalize_routing.cpp:943-1083): the reference's route for INT8 weights.
+extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNzGetWorkspaceSize(
+    const aclTensor* x1, const aclTensor* x2, const aclTensor* scale, const aclTensor* bias,
+    const aclTensor* pertokenScaleOptional, const aclTensor* groupList, const aclTensor* sharedInput, const aclTensor* logit,
+    const aclTensor* rowIndex, int64_t dtype, float sharedInputWeight, int64_t sharedInputOffset, bool transposeX1,
+    bool transposeX2, int64_t groupListType, aclTensor* out, uint64_t* workspaceSize, aclOpExecutor** executor) {
+    return PlanCombine("GroupedMatmulFinalizeRoutingWeightNz", x1, x2, scale, bias, nullptr, nullptr, nullptr,
+                       pertokenScaleOptional, groupList, sharedInput, logit, rowIndex, dtype, sharedInputWeight,
+                       sharedInputOffset, transposeX1, transposeX2, groupListType, nullptr, /*forceNz=*/true, out,
+                       workspaceSize, executor);
+}
+
+extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNz(void* workspace, uint64_t workspaceSize,
+                                                                 aclOpExecutor* executor, aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
+}
+
+extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNzV2GetWorkspaceSize(
+    const aclTensor* x1, aclTensor* x2, const aclTensor* scale, const aclTensor* bias, const aclTensor* offsetOptional,
+    const aclTensor* antiquantScaleOptional, const aclTensor* antiquantOffsetOptional,
+    const aclTensor* pertokenScaleOptional, const aclTensor* groupList, const aclTensor* sharedInput, const aclTensor* logit,
+    const aclTensor* rowIndex, int64_t dtype, float sharedInputWeight, int64_t sharedInputOffset, bool transposeX1,
+    bool transposeX2, int64_t groupListType, const aclIntArray* tuningConfigOptional, aclTensor* out,
+    uint64_t* workspaceSize, aclOpExecutor** executor) {
+    return PlanCombine("GroupedMatmulFinalizeRoutingWeightNzV2", x1, x2, scale, bias, offsetOptional, antiquantScaleOptional,
+                       antiquantOffsetOptional, pertokenScaleOptional, groupList, sharedInput, logit, rowIndex, dtype,
+                       sharedInputWeight, sharedInputOffset, transposeX1, transposeX2, groupListType, tuningConfigOptional,
+                       /*forceNz=*/true, out, workspaceSize, executor);
+}
+
+extern "C" aclnnStatus aclnnGroupedMatmulFinalizeRoutingWeightNzV2(void* workspace, uint64_t workspaceSize,
+                                                                   aclOpExecutor* executor, aclrtStream stream) {
     return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
 }

@@ -3,11 +3,14 @@
 // Argument checks follow gmm/grouped_matmul_swiglu_quant/op_host/op_api/aclnn_grouped_matmul_swiglu_quant.cpp:75-350,
 // 365-409 (required tensors, ranks, shapes, dtypes, groupList length <= E, K < 65536, N even) and :425-429 (an empty
 // output / groupList / outputScale succeeds with no work).  The N <= 10240 ceiling and the FRACTAL_NZ-only weight rule
-// of the reference are not carried over.  The arithmetic is in grouped_gemm_i8.hip (kSwiglu epilogue + requantisation).
+// of the reference are not carried over: ND weights are taken as well.  A FRACTAL_NZ weight is the 5-D tensor
+// [E, N/32, K/16, 16, 32] (:163-181), or through aclnnGroupedMatmulSwigluQuantWeightNZ any tensor whose storage shape
+// is that (:483-516).  The arithmetic is in grouped_gemm_i8.hip (kSwiglu epilogue + requantisation).
 //
 // All state lives in the executor; the reference's two sticky file-scope switches
 // (aclnn_grouped_matmul_swiglu_quant.cpp:61-62) have no counterpart here.
 #include "aclnnop/aclnn_grouped_matmul_swiglu_quant.h"
+#include "aclnnop/aclnn_grouped_matmul_swiglu_quant_weight_nz.h"
 
 #include <new>
 
@@ -37,12 +40,11 @@ class SwigluQuantExecutor : public aclOpExecutor {
 
 constexpr int64_t kKLimit = 65536;
 
-}  // namespace
-
-extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantGetWorkspaceSize(
-    const aclTensor* x, const aclTensor* weight, const aclTensor* bias, const aclTensor* offset,
-    const aclTensor* weightScale, const aclTensor* xScale, const aclTensor* groupList, aclTensor* output,
-    aclTensor* outputScale, aclTensor* outputOffset, uint64_t* workspaceSize, aclOpExecutor** executor) {
+// forceNz: the WeightNZ entry point, where the storage is blocked whatever the descriptor's format field says.
+aclnnStatus PlanSwigluQuant(const aclTensor* x, const aclTensor* weight, const aclTensor* bias, const aclTensor* offset,
+                            const aclTensor* weightScale, const aclTensor* xScale, const aclTensor* groupList,
+                            aclTensor* output, aclTensor* outputScale, aclTensor* outputOffset, bool forceNz,
+                            uint64_t* workspaceSize, aclOpExecutor** executor) {
     using namespace opapi;
     ClearError();
     (void)bias;          // accepted and ignored, as in the reference's A8W8 path (only a warning there)
@@ -61,10 +63,22 @@ extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantGetWorkspaceSize(
 
     OPAPI_CHECK(x->dtype == ACL_INT8 && weight->dtype == ACL_INT8, kInvalid,
                 "only the A8W8 path is built: x and weight must be INT8 (got %d, %d)", (int)x->dtype, (int)weight->dtype);
-    OPAPI_CHECK(weight->format == ACL_FORMAT_ND, kInvalid,
-                "weight must be ND (row-major [E,K,N] or its transposed-storage view); FRACTAL_NZ is not accepted");
+    const bool nz = forceNz || weight->format == ACL_FORMAT_FRACTAL_NZ;
+    OPAPI_CHECK(nz || weight->format == ACL_FORMAT_ND, kInvalid, "weight Format expect is ND or FRACTAL_NZ, but got [%d].",
+                (int)weight->format);
     OPAPI_CHECK(x->dims.size() == 2, kInvalid, "x must be 2-D [M,K], got %s", ShapeStr(x).c_str());
-    OPAPI_CHECK(weight->dims.size() == 3, kInvalid, "weight must be 3-D [E,K,N], got %s", ShapeStr(weight).c_str());
+    // a blocked weight is described either by its 5-D shape [E, N/32, K/16, 16, 32] or by the 3-D view [E, K, N] over
+    // storage of that shape
+    const std::vector<int64_t>& blocked = weight->dims.size() == 5 ? weight->dims : weight->storage;
+    if (nz) {
+        OPAPI_CHECK(weight->dims.size() == 5 || weight->dims.size() == 3, kInvalid,
+                    "a FRACTAL_NZ weight must be 5-D [E,N/32,K/16,16,32] or a 3-D view of such storage, got %s",
+                    ShapeStr(weight).c_str());
+        OPAPI_CHECK(blocked.size() == 5 && blocked[3] == 16 && blocked[4] == 32, kInvalid,
+                    "The dimnum of storageShape for second input (weight) must be 5 with the last two dims (16, 32).");
+    } else {
+        OPAPI_CHECK(weight->dims.size() == 3, kInvalid, "weight must be 3-D [E,K,N], got %s", ShapeStr(weight).c_str());
+    }
     OPAPI_CHECK(weightScale->dims.size() == 2, kInvalid, "weightScale must be 2-D [E,N], got %s",
                 ShapeStr(weightScale).c_str());
     OPAPI_CHECK(xScale->dims.size() == 1, kInvalid, "xScale must be 1-D [M], got %s", ShapeStr(xScale).c_str());
@@ -73,9 +87,15 @@ extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantGetWorkspaceSize(
     OPAPI_CHECK(outputScale->dims.size() == 1, kInvalid, "outputScale must be 1-D [M], got %s",
                 ShapeStr(outputScale).c_str());
 
-    const int64_t e = weight->dims[0], m = x->dims[0], k = x->dims[1], n = weight->dims[2];
-    OPAPI_CHECK(weight->dims[1] == k, kInvalid, "weight %s does not match x %s along K", ShapeStr(weight).c_str(),
-                ShapeStr(x).c_str());
+    const int64_t e = weight->dims[0], m = x->dims[0], k = x->dims[1];
+    const int64_t n = weight->dims.size() == 5 ? weight->dims[1] * 32 : weight->dims[2];
+    const int64_t wk = weight->dims.size() == 5 ? weight->dims[2] * 16 : weight->dims[1];
+    OPAPI_CHECK(wk == k, kInvalid, "weight %s does not match x %s along K", ShapeStr(weight).c_str(), ShapeStr(x).c_str());
+    if (nz) {
+        OPAPI_CHECK(blocked[0] == e && blocked[1] * 32 == n && blocked[2] * 16 == k, kInvalid,
+                    "the blocked weight storage must be [%lld, %lld, %lld, 16, 32] (N a multiple of 32, K of 16)",
+                    (long long)e, (long long)(n / 32), (long long)(k / 16));
+    }
     OPAPI_CHECK(n % 2 == 0, kInvalid, "N is %lld , which must even number.", (long long)n);
     OPAPI_CHECK(weightScale->dims[0] == e && weightScale->dims[1] == n, kInvalid, "weightScale must be [%lld,%lld], got %s",
                 (long long)e, (long long)n, ShapeStr(weightScale).c_str());
@@ -109,9 +129,10 @@ extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantGetWorkspaceSize(
     }
     OPAPI_CHECK(k > 0, kInvalid, "K must be positive");
 
-    const bool wTransposed = IsLastTwoDimsTransposed(weight);
-    OPAPI_CHECK(wTransposed || IsContiguous(weight), kInvalid,
+    const bool wTransposed = !nz && IsLastTwoDimsTransposed(weight);
+    OPAPI_CHECK(nz || wTransposed || IsContiguous(weight), kInvalid,
                 "weight must be contiguous [E,K,N] or the transposed view of contiguous [E,N,K] storage");
+    OPAPI_CHECK(!nz || weight->offset == 0, kInvalid, "a FRACTAL_NZ weight must start at its storage");
     OPAPI_CHECK(IsContiguous(x) && IsContiguous(weightScale) && IsContiguous(xScale) && IsContiguous(groupList) &&
                     IsContiguous(output) && IsContiguous(outputScale),
                 kInvalid, "x, weightScale, xScale, groupList, output and outputScale must be contiguous");
@@ -126,6 +147,7 @@ extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantGetWorkspaceSize(
     p.x = reinterpret_cast<const int8_t*>(DataPtr(x));
     p.w = reinterpret_cast<const int8_t*>(DataPtr(weight));
     p.wKMajor = wTransposed;
+    p.wNz = nz;
     p.M = m;
     p.K = k;
     p.N = n;
@@ -144,6 +166,29 @@ extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantGetWorkspaceSize(
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantGetWorkspaceSize(
+    const aclTensor* x, const aclTensor* weight, const aclTensor* bias, const aclTensor* offset,
+    const aclTensor* weightScale, const aclTensor* xScale, const aclTensor* groupList, aclTensor* output,
+    aclTensor* outputScale, aclTensor* outputOffset, uint64_t* workspaceSize, aclOpExecutor** executor) {
+    return PlanSwigluQuant(x, weight, bias, offset, weightScale, xScale, groupList, output, outputScale, outputOffset,
+                           /*forceNz=*/false, workspaceSize, executor);
+}
+
+extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantWeightNZGetWorkspaceSize(
+    const aclTensor* x, const aclTensor* weight, const aclTensor* bias, const aclTensor* offset,
+    const aclTensor* weightScale, const aclTensor* xScale, const aclTensor* groupList, aclTensor* output,
+    aclTensor* outputScale, aclTensor* outputOffset, uint64_t* workspaceSize, aclOpExecutor** executor) {
+    return PlanSwigluQuant(x, weight, bias, offset, weightScale, xScale, groupList, output, outputScale, outputOffset,
+                           /*forceNz=*/true, workspaceSize, executor);
+}
+
+extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuantWeightNZ(void* workspace, uint64_t workspaceSize,
+                                                             aclOpExecutor* executor, aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
 }
 
 extern "C" aclnnStatus aclnnGroupedMatmulSwigluQuant(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,

@@ -12,6 +12,7 @@
 // Widenings of this build: scale FLOAT with out BF16 is accepted; groupList may be INT32.
 // Group boundaries: grouped_matmul_utils.h:243-257.  The arithmetic is in grouped_gemm_i8.hip.
 #include "aclnnop/aclnn_grouped_matmul_v5.h"
+#include "aclnnop/aclnn_grouped_matmul_weight_nz.h"
 
 #include <new>
 
@@ -66,8 +67,8 @@ aclnnStatus PlanGroupedMatmul(
     const aclTensor* groupListOptional, const aclTensorList* activationInputOptional,
     const aclTensorList* activationQuantScaleOptional, const aclTensorList* activationQuantOffsetOptional,
     int64_t splitItem, int64_t groupType, int64_t groupListType, int64_t actType, int64_t expectedRowsPerGroup,
-    aclTensorList* out, aclTensorList* activationFeatureOutOptional, aclTensorList* dynQuantScaleOutOptional,
-    uint64_t* workspaceSize, aclOpExecutor** executor) {
+    bool forceNz, aclTensorList* out, aclTensorList* activationFeatureOutOptional,
+    aclTensorList* dynQuantScaleOutOptional, uint64_t* workspaceSize, aclOpExecutor** executor) {
     using namespace opapi;
     ClearError();
     constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;
@@ -122,7 +123,16 @@ aclnnStatus PlanGroupedMatmul(
     OPAPI_CHECK(yt != nullptr, kInvalid, "y[0] is nullptr!");
     OPAPI_CHECK(xt->dtype == ACL_INT8 && wt->dtype == ACL_INT8, kInvalid,
                 "only INT8 x and INT8 weight are built (got %d, %d)", (int)xt->dtype, (int)wt->dtype);
-    OPAPI_CHECK(wt->format == ACL_FORMAT_ND, kInvalid, "weight must be ND");
+    // A blocked (FRACTAL_NZ) int8 weight is [E, N/32, K/16, 16, 32], given as that 5-D tensor or as the 3-D view
+    // [E, K, N] over storage of that shape (the layout aclnn_grouped_matmul_swiglu_quant.cpp:163-168 spells out).
+    const bool nz = forceNz || wt->format == ACL_FORMAT_FRACTAL_NZ;
+    OPAPI_CHECK(nz || wt->format == ACL_FORMAT_ND, kInvalid, "weight must be ND or FRACTAL_NZ");
+    const std::vector<int64_t>& blocked = wt->dims.size() == 5 ? wt->dims : wt->storage;
+    if (nz) {
+        OPAPI_CHECK((wt->dims.size() == 5 || wt->dims.size() == 3) && blocked.size() == 5 && blocked[3] == 16 && blocked[4] == 32,
+                    kInvalid, "a FRACTAL_NZ weight needs the storage shape [E, N/32, K/16, 16, 32], got view %s",
+                    ShapeStr(wt).c_str());
+    }
     OPAPI_CHECK(actType == GMM_ACT_TYPE_NONE, kInvalid, "actType %lld is not built for the INT8 path", (long long)actType);
     OPAPI_CHECK(!Present(biasOptional), kInvalid, "bias is not supported on the INT8 per-token path of this build");
     OPAPI_CHECK(!Present(offsetOptional), kInvalid, "offset must be null in the quant case");
@@ -130,11 +140,15 @@ aclnnStatus PlanGroupedMatmul(
                 "antiquant parameters must be null in the quant case");
 
     OPAPI_CHECK(xt->dims.size() == 2, kInvalid, "x must be 2-D [M,K], got %s", ShapeStr(xt).c_str());
-    OPAPI_CHECK(wt->dims.size() == 3, kInvalid, "weight must be 3-D [E,K,N], got %s", ShapeStr(wt).c_str());
+    OPAPI_CHECK(nz || wt->dims.size() == 3, kInvalid, "weight must be 3-D [E,K,N], got %s", ShapeStr(wt).c_str());
     OPAPI_CHECK(yt->dims.size() == 2, kInvalid, "y must be 2-D [M,N], got %s", ShapeStr(yt).c_str());
-    const int64_t m = xt->dims[0], k = xt->dims[1], e = wt->dims[0], n = wt->dims[2];
-    OPAPI_CHECK(wt->dims[1] == k, kInvalid, "weight %s does not match x %s along K", ShapeStr(wt).c_str(),
-                ShapeStr(xt).c_str());
+    const int64_t m = xt->dims[0], k = xt->dims[1], e = wt->dims[0];
+    const int64_t n = wt->dims.size() == 5 ? wt->dims[1] * 32 : wt->dims[2];
+    const int64_t wk = wt->dims.size() == 5 ? wt->dims[2] * 16 : wt->dims[1];
+    OPAPI_CHECK(wk == k, kInvalid, "weight %s does not match x %s along K", ShapeStr(wt).c_str(), ShapeStr(xt).c_str());
+    OPAPI_CHECK(!nz || (blocked[0] == e && blocked[1] * 32 == n && blocked[2] * 16 == k && wt->offset == 0), kInvalid,
+                "the blocked weight storage must be [%lld, %lld, %lld, 16, 32] (N a multiple of 32, K of 16)", (long long)e,
+                (long long)(n / 32), (long long)(k / 16));
     OPAPI_CHECK(yt->dims[0] == m && yt->dims[1] == n, kInvalid, "y must be [%lld,%lld], got %s", (long long)m, (long long)n,
                 ShapeStr(yt).c_str());
     OPAPI_CHECK(k < 65536, kInvalid, "K must be lower than 65536");
@@ -182,8 +196,8 @@ aclnnStatus PlanGroupedMatmul(
     }
     OPAPI_CHECK(k > 0, kInvalid, "K must be positive");
 
-    const bool wTransposed = IsLastTwoDimsTransposed(wt);
-    OPAPI_CHECK(wTransposed || IsContiguous(wt), kInvalid,
+    const bool wTransposed = !nz && IsLastTwoDimsTransposed(wt);
+    OPAPI_CHECK(nz || wTransposed || IsContiguous(wt), kInvalid,
                 "weight must be contiguous [E,K,N] or the transposed view of contiguous [E,N,K] storage");
     OPAPI_CHECK(IsContiguous(xt) && IsContiguous(yt) && IsContiguous(groupListOptional), kInvalid,
                 "x, y and groupList must be contiguous");
@@ -200,6 +214,7 @@ aclnnStatus PlanGroupedMatmul(
     p.x = reinterpret_cast<const int8_t*>(DataPtr(xt));
     p.w = reinterpret_cast<const int8_t*>(DataPtr(wt));
     p.wKMajor = wTransposed;
+    p.wNz = nz;
     p.M = m;
     p.K = k;
     p.N = n;
@@ -240,7 +255,7 @@ extern "C" aclnnStatus aclnnGroupedMatmulV4GetWorkspaceSize(
     return PlanGroupedMatmul(x, weight, biasOptional, scaleOptional, offsetOptional, antiquantScaleOptional,
                              antiquantOffsetOptional, perTokenScaleOptional, groupListOptional, activationInputOptional,
                              activationQuantScaleOptional, activationQuantOffsetOptional, splitItem, groupType,
-                             groupListType, actType, /*expectedRowsPerGroup=*/0, out, activationFeatureOutOptional,
+                             groupListType, actType, /*expectedRowsPerGroup=*/0, /*forceNz=*/false, out, activationFeatureOutOptional,
                              dynQuantScaleOutOptional, workspaceSize, executor);
 }
 
@@ -263,7 +278,7 @@ extern "C" aclnnStatus aclnnGroupedMatmulV5GetWorkspaceSize(
     return PlanGroupedMatmul(x, weight, biasOptional, scaleOptional, offsetOptional, antiquantScaleOptional,
                              antiquantOffsetOptional, perTokenScaleOptional, groupListOptional, activationInputOptional,
                              activationQuantScaleOptional, activationQuantOffsetOptional, splitItem, groupType,
-                             groupListType, actType, expected, out, activationFeatureOutOptional,
+                             groupListType, actType, expected, /*forceNz=*/false, out, activationFeatureOutOptional,
                              dynQuantScaleOutOptional, workspaceSize, executor);
 }
 
@@ -274,5 +289,39 @@ extern "C" aclnnStatus aclnnGroupedMatmulV5(void* workspace, uint64_t workspaceS
 
 extern "C" aclnnStatus aclnnGroupedMatmulV4(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
                                             aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
+}
+
+// V5 for a weight whose storage is the blocked FRACTAL_NZ layout, plus quantGroupSize (per-group quantisation: must be 0
+// here) -- reference: aclnn_grouped_matmul.cpp:1918-1956.
+extern "C" aclnnStatus aclnnGroupedMatmulWeightNzGetWorkspaceSize(
+    const aclTensorList* x, const aclTensorList* weight, const aclTensorList* biasOptional,
+    const aclTensorList* scaleOptional, const aclTensorList* offsetOptional, const aclTensorList* antiquantScaleOptional,
+    const aclTensorList* antiquantOffsetOptional, const aclTensorList* perTokenScaleOptional,
+    const aclTensor* groupListOptional, const aclTensorList* activationInputOptional,
+    const aclTensorList* activationQuantScaleOptional, const aclTensorList* activationQuantOffsetOptional,
+    int64_t splitItem, int64_t groupType, int64_t groupListType, int64_t actType, aclIntArray* tuningConfigOptional,
+    int64_t quantGroupSize, aclTensorList* out, aclTensorList* activationFeatureOutOptional,
+    aclTensorList* dynQuantScaleOutOptional, uint64_t* workspaceSize, aclOpExecutor** executor) {
+    if (quantGroupSize != 0) {
+        opapi::ClearError();
+        opapi::SetError("aclnnGroupedMatmulWeightNz: per-group quantisation (quantGroupSize %lld) is not built; pass 0",
+                        (long long)quantGroupSize);
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    int64_t expected = 0;
+    if (tuningConfigOptional != nullptr && !tuningConfigOptional->values.empty() &&
+        tuningConfigOptional->values[0] > 0) {
+        expected = tuningConfigOptional->values[0];
+    }
+    return PlanGroupedMatmul(x, weight, biasOptional, scaleOptional, offsetOptional, antiquantScaleOptional,
+                             antiquantOffsetOptional, perTokenScaleOptional, groupListOptional, activationInputOptional,
+                             activationQuantScaleOptional, activationQuantOffsetOptional, splitItem, groupType,
+                             groupListType, actType, expected, /*forceNz=*/true, out, activationFeatureOutOptional,
+                             dynQuantScaleOutOptional, workspaceSize, executor);
+}
+
+extern "C" aclnnStatus aclnnGroupedMatmulWeightNz(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
+                                                  aclrtStream stream) {
     return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
 }

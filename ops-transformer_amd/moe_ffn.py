@@ -33,11 +33,17 @@ class MoeFfnW8A8:
     The operators see the reference layout [E, K, N] through transposed views of this storage.
     """
 
-    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v3", fused_combine=False):
+    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v3", fused_combine=False,
+                 weight_nz=False):
         assert routing in ("v2", "v3")
         assert not (fused_combine and routing != "v3")
+        assert not (fused_combine and weight_nz)
         self.routing = routing
         self.fused_combine = fused_combine
+        # weight_nz: hand the operators the reference's FRACTAL_NZ weights ([E, N/32, K/16, 16, 32]) instead of the
+        # transposed views; the blocked copies are made here, once
+        self.w13_nz = self.to_nz(w13) if weight_nz else None
+        self.w2_nz = self.to_nz(w2) if weight_nz else None
         assert w13.dtype == torch.int8 and w2.dtype == torch.int8
         self.w13_view = w13.transpose(1, 2)  # [E, H, 2I]
         self.w2_view = w2.transpose(1, 2)    # [E, I, H]
@@ -49,6 +55,12 @@ class MoeFfnW8A8:
         self.out_dtype = out_dtype
         self.device = w13.device
         self._buf_key = None
+
+    @staticmethod
+    def to_nz(w_enk):
+        """K-contiguous storage [E, N, K] -> blocked [E, N/32, K/16, 16, 32] (element (k, n) at [n/32][k/16][k%16][n%32])."""
+        E, N, K = w_enk.shape
+        return w_enk.view(E, N // 32, 32, K // 16, 16).permute(0, 1, 3, 4, 2).contiguous()
 
     def _buffers(self, T, K):
         if self._buf_key == (T, K):
@@ -84,8 +96,9 @@ class MoeFfnW8A8:
             aclnn.moe_init_routing_v2(x_scale.view(T, 1), topk_idx, 0, 0, E, 0, 0, False,
                                       out=(self.expanded_scale.view(T * K, 1), self.row_idx_scratch, None, None),
                                       workspace=self.workspace)
-        aclnn.grouped_matmul_swiglu_quant(self.expanded_x, self.w13_view, self.cumsum, self.w13_scale,
-                                          self.expanded_scale, out=(self.h, self.h_scale),
+        aclnn.grouped_matmul_swiglu_quant(self.expanded_x, None if self.w13_nz is not None else self.w13_view, self.cumsum,
+                                          self.w13_scale, self.expanded_scale, out=(self.h, self.h_scale),
+                                          weight_nz=None if self.w13_nz is None else (self.w13_nz, "nz5d"),
                                           workspace=self.workspace)
         if self.fused_combine:
             source = self.expanded_row_idx.long()                       # expanded row -> flat (token, k) position
@@ -94,7 +107,9 @@ class MoeFfnW8A8:
                                                   group_list_type=0, per_token_scale=self.h_scale, logit=logit,
                                                   out=self.out, workspace=self.workspace)
             return self.out
-        aclnn.grouped_matmul_v4([self.h], [self.w2_view], scale=[self.w2_scale], per_token_scale=[self.h_scale],
+        aclnn.grouped_matmul_v4([self.h], None if self.w2_nz is not None else [self.w2_view],
+                                weight_nz=None if self.w2_nz is None else (self.w2_nz, "nz5d"),
+                                scale=[self.w2_scale], per_token_scale=[self.h_scale],
                                 group_list=self.cumsum, split_item=3, group_type=0, group_list_type=0, act_type=0,
                                 out=[self.y], workspace=self.workspace)
         aclnn.moe_finalize_routing_v2(self.y, self.expanded_row_idx, scales=topk_weight, drop_pad_mode=2, out=self.out)

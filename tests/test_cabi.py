@@ -35,7 +35,12 @@ def test_headers_declare_the_expected_entry_points():
                      "aclnnGroupedMatmulFinalizeRoutingGetWorkspaceSize", "aclnnGroupedMatmulFinalizeRouting",
                      "aclnnGroupedMatmulFinalizeRoutingV2GetWorkspaceSize", "aclnnGroupedMatmulFinalizeRoutingV2",
                      "aclnnGroupedMatmulFinalizeRoutingV3GetWorkspaceSize", "aclnnGroupedMatmulFinalizeRoutingV3",
+                     "aclnnGroupedMatmulFinalizeRoutingWeightNzGetWorkspaceSize", "aclnnGroupedMatmulFinalizeRoutingWeightNz",
+                     "aclnnGroupedMatmulFinalizeRoutingWeightNzV2GetWorkspaceSize",
+                     "aclnnGroupedMatmulFinalizeRoutingWeightNzV2",
                      "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize", "aclnnGroupedMatmulSwigluQuant",
+                     "aclnnGroupedMatmulSwigluQuantWeightNZGetWorkspaceSize", "aclnnGroupedMatmulSwigluQuantWeightNZ",
+                     "aclnnGroupedMatmulWeightNzGetWorkspaceSize", "aclnnGroupedMatmulWeightNz",
                      "aclnnGroupedMatmulV4GetWorkspaceSize", "aclnnGroupedMatmulV4",
                      "aclnnGroupedMatmulV5GetWorkspaceSize", "aclnnGroupedMatmulV5",
                      "aclnnMoeFinalizeRoutingV2GetWorkspaceSize", "aclnnMoeFinalizeRoutingV2",
@@ -59,9 +64,9 @@ class T:
     """Descriptor over a fake device address (phase 1 never dereferences it)."""
     _next = 0x10000
 
-    def __init__(self, aclnn, shape, dtype, strides=None, data=True, fmt=2):
+    def __init__(self, aclnn, shape, dtype, strides=None, data=True, fmt=2, storage=None):
         T._next += 0x10000
-        self.h = aclnn.create_tensor(list(shape), dtype, T._next if data else 0, strides, 0, fmt)
+        self.h = aclnn.create_tensor(list(shape), dtype, T._next if data else 0, strides, 0, fmt, storage)
 
 
 def _status(aclnn, api, args):
@@ -259,7 +264,8 @@ def test_routing_v3_nulls(aclnn):
 # ------------------------------------------------------------------------------------------------ SwiGLU quant
 def _swiglu_args(aclnn, M=192, K=2048, N=2048, E=4, **over):
     x = T(aclnn, over.get("x_shape", (M, K)), over.get("x_dtype", I8))
-    w = T(aclnn, over.get("w_shape", (E, K, N)), over.get("w_dtype", I8), over.get("w_strides"), fmt=over.get("w_fmt", 2))
+    w = T(aclnn, over.get("w_shape", (E, K, N)), over.get("w_dtype", I8), over.get("w_strides"), fmt=over.get("w_fmt", 2),
+          storage=over.get("w_storage"))
     ws = T(aclnn, over.get("ws_shape", (E, N)), over.get("ws_dtype", F32))
     xs = T(aclnn, over.get("xs_shape", (M,)), F32)
     gl = T(aclnn, (over.get("gl_len", E),), over.get("gl_dtype", I64))
@@ -280,7 +286,11 @@ def test_swiglu_valid(aclnn):
 
 @pytest.mark.parametrize("kw,fragment", [
     (dict(x_dtype=F16), "A8W8"),
-    (dict(w_fmt=29), "FRACTAL_NZ"),
+    (dict(w_fmt=29), "storageShape for second input (weight) must be 5"),          # NZ format over plain 3-D storage
+    (dict(w_fmt=29, w_shape=(4, 64, 128, 16, 16)), "last two dims (16, 32)"),
+    (dict(w_fmt=29, w_shape=(4, 64, 127, 16, 32)), "does not match x"),
+    (dict(w_fmt=29, w_storage=(4, 64, 127, 16, 32)), "blocked weight storage must be [4, 64, 128, 16, 32]"),
+    (dict(w_fmt=4), "ND or FRACTAL_NZ"),
     (dict(N=2047, out_shape=(192, 1023), ws_shape=(4, 2047)), "must even number"),
     (dict(ws_shape=(4, 2046)), "weightScale must be"),
     (dict(xs_shape=(191,)), "xScale must be"),
@@ -293,6 +303,20 @@ def test_swiglu_valid(aclnn):
 def test_swiglu_invalid(aclnn, kw, fragment):
     code, msg = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, **kw))
     assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_swiglu_nz_weight_forms(aclnn):
+    """The FRACTAL_NZ weight of the reference: 5-D [E, N/32, K/16, 16, 32], or a 3-D view over such storage; through the
+    WeightNZ entry point the format field does not matter but the storage shape must be the blocked one."""
+    nz5 = dict(w_fmt=29, w_shape=(4, 64, 128, 16, 32))
+    nz3 = dict(w_fmt=29, w_storage=(4, 64, 128, 16, 32))
+    for api, kw in [("aclnnGroupedMatmulSwigluQuant", nz5), ("aclnnGroupedMatmulSwigluQuant", nz3),
+                    ("aclnnGroupedMatmulSwigluQuantWeightNZ", dict(nz5, w_fmt=2)),
+                    ("aclnnGroupedMatmulSwigluQuantWeightNZ", dict(nz3, w_fmt=2))]:
+        code, ws = _status(aclnn, api, _swiglu_args(aclnn, **kw))
+        assert code == 0, (api, kw, ws)
+    code, msg = _status(aclnn, "aclnnGroupedMatmulSwigluQuantWeightNZ", _swiglu_args(aclnn))     # plain ND storage
+    assert code == INVALID and "storageShape" in msg
 
 
 def test_swiglu_null_and_empty(aclnn):
@@ -428,7 +452,8 @@ def test_combine_valid(aclnn):
     (dict(tx=True), "transpose should be false"),
     (dict(tw=True), "transpose should be false"),
     (dict(w_dtype=I32, w_shape=(4, 256, 16)), "INT4 weights"),
-    (dict(w_fmt=29), "format should be ND"),
+    (dict(w_fmt=29), "x2's format is not NZ"),                     # NZ format over plain 3-D storage
+    (dict(w_fmt=4), "format should be ND or FRACTAL_NZ"),
     (dict(x_dtype=BF16), "x1 must be INT8"),
     (dict(scale_dtype=I64), "scale must be FLOAT or BF16"),
     (dict(scale_shape=(3, 128)), "Scale fisrt dim should equal to weight EDim 4, but actual is 3"),

@@ -112,3 +112,21 @@ def test_fused_chain_matches_unfused_chain(pkg, dev):
     assert fused.dtype == torch.float32
     err = (fused - plain).abs().max().item()
     assert err <= 2e-2 * plain.abs().max().item(), err
+
+
+@pytest.mark.parametrize("version", [1, 2])
+def test_weight_nz_entry_points(aclnn, oracle, dev, version):
+    """aclnnGroupedMatmulFinalizeRoutingWeightNz / WeightNzV2: the blocked weight gives what the ND weight gives (to the
+    bound of the atomic order) and agrees with the oracle."""
+    rng = np.random.default_rng(20 + version)
+    M, K, N, E, batch, topk = 300, 512, 544, 7, 75, 4
+    x, w, cumsum, scale, pt, logit, row_index = _case(rng, M, K, N, E, batch, topk)
+    w_nz = np.ascontiguousarray(w.reshape(E, N // 32, 32, K // 16, 16).transpose(0, 1, 3, 4, 2))   # from [E, N, K] storage
+    t = lambda a: torch.from_numpy(a).to(dev)
+    counts = np.diff(np.concatenate([[0], cumsum])).astype(np.int64)
+    out = aclnn.grouped_matmul_finalize_routing(t(x), None, t(scale), t(row_index), batch, t(counts), group_list_type=1,
+                                                per_token_scale=t(pt), logit=t(logit), version=version, weight_nz=t(w_nz))
+    torch.cuda.synchronize()
+    ref = oracle.grouped_matmul_finalize_routing(x, w, scale, row_index, batch, counts, list_type=1, w_trans=True,
+                                                 per_token=pt, logit=logit)
+    assert np.abs(out.cpu().numpy() - ref).max() <= _tolerance(oracle, x, w, cumsum, scale, pt, logit)

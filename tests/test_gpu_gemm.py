@@ -270,3 +270,62 @@ def test_sparse_list_from_routing_v3(aclnn, oracle, dev):
     ex_r, _, cnt_r, _ = oracle.moe_init_routing_v3(x, idx, None, E, None, 1, 1)
     ref = oracle.grouped_matmul_i32(ex_r, wt, cnt_r, list_type=1, w_trans=True)
     assert np.array_equal(out.cpu().numpy(), ref)
+
+
+# ------------------------------------------------------------------------------------------------ FRACTAL_NZ weights
+def _to_nz(w_ekn):
+    """[E, K, N] -> the blocked layout [E, N/32, K/16, 16, 32]: element (k, n) at [n / 32][k / 16][k % 16][n % 32]."""
+    E, K, N = w_ekn.shape
+    return np.ascontiguousarray(w_ekn.reshape(E, K // 16, 16, N // 32, 32).transpose(0, 3, 1, 2, 4))
+
+
+NZ_CASES = [  # M, K, N, E, mode, how
+    (37, 128, 64, 4, "ragged", "nz5d"),            # N/2 = 32: one channel block per half
+    (96, 256, 320, 7, "ragged", "entry5d"),        # partial n-tile
+    (512, 1024, 512, 8, "even", "entry3d"),
+    (512, 4096, 3072, 128, "ragged", "nz5d"),      # decode shape
+    (700, 512, 576, 3, "ragged", "nz5d"),          # 256-row tiles
+    (300, 208, 128, 4, "ragged", "nz5d"),          # K not a multiple of 128: byte-wise kernel
+    (2048, 2048, 512, 16, "even", "entry5d"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,E,mode,how", NZ_CASES)
+def test_swiglu_quant_nz_weight_equals_nd_weight(aclnn, oracle, dev, M, K, N, E, mode, how):
+    """The blocked weight layout gives exactly what the same weights give as an ND tensor (same arithmetic, other
+    addressing), and that stays within the operator's bars against the oracle."""
+    rng = np.random.default_rng(M + K + N)
+    x, wt, cumsum = _problem(rng, M, K, N, E, mode)            # wt: [E, N, K] storage
+    w_ekn = np.ascontiguousarray(wt.transpose(0, 2, 1))
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    xs = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    q_nd, s_nd = aclnn.grouped_matmul_swiglu_quant(t(x), t(wt).transpose(1, 2), t(cumsum), t(scale), t(xs))
+    q_nz, s_nz = aclnn.grouped_matmul_swiglu_quant(t(x), None, t(cumsum), t(scale), t(xs), weight_nz=(t(_to_nz(w_ekn)), how))
+    torch.cuda.synchronize()
+    rows = int(cumsum[-1])
+    assert torch.equal(q_nd[:rows], q_nz[:rows]) and torch.equal(s_nd[:rows], s_nz[:rows])
+    ref_q, ref_s = oracle.grouped_matmul_swiglu_quant(x, wt, scale, xs, cumsum, w_trans=True)
+    assert np.abs(q_nz.cpu().numpy()[:rows].astype(np.int32) - ref_q[:rows].astype(np.int32)).max() <= 1
+    np.testing.assert_allclose(s_nz.cpu().numpy()[:rows], ref_s[:rows], rtol=1e-2)
+
+
+@pytest.mark.parametrize("M,K,N,E,mode,how", [(37, 128, 64, 4, "ragged", "nz5d"), (96, 256, 320, 7, "ragged", "entry5d"),
+                                              (512, 1024, 512, 8, "even", "entry3d"), (700, 512, 544, 3, "ragged", "nz5d"),
+                                              (300, 208, 96, 4, "ragged", "entry3d"), (512, 1536, 4096, 128, "ragged", "nz5d")])
+def test_grouped_matmul_nz_weight(aclnn, oracle, dev, M, K, N, E, mode, how):
+    """int32 accumulators and the bf16 down-projection output with a blocked weight: bit-exact against the oracle."""
+    rng = np.random.default_rng(M + K + N + 1)
+    x, wt, cumsum = _problem(rng, M, K, N, E, mode)
+    w_nz = torch.from_numpy(_to_nz(np.ascontiguousarray(wt.transpose(0, 2, 1)))).to(dev)
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    acc = aclnn.grouped_matmul_v4([t(x)], None, group_list=t(cumsum), split_item=3, group_type=0, weight_nz=(w_nz, how))[0]
+    y = aclnn.grouped_matmul_v4([t(x)], None, scale=[t(scale)], per_token_scale=[t(pt)], group_list=t(cumsum), split_item=3,
+                                group_type=0, output_dtype=torch.bfloat16, weight_nz=(w_nz, how), tuning_config=[M // E])[0]
+    torch.cuda.synchronize()
+    rows = int(cumsum[-1])
+    assert np.array_equal(acc.cpu().numpy()[:rows], oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)[:rows])
+    ref = oracle.grouped_matmul_dequant(x, wt, scale, pt, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16)[:rows], ref[:rows])

@@ -113,3 +113,16 @@ def test_graph_replays_match_eager(pkg, dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.int16), want.view(torch.int16)), seed
+
+
+def test_nz_weight_chain_equals_nd_chain(pkg, dev):
+    """The chain fed FRACTAL_NZ weights equals the chain fed the transposed views, bit for bit."""
+    cfg = pkg.synth.config(0)
+    idx, wgt = pkg.synth.make_routing(cfg, seed=0)
+    xq, xs = pkg.synth.make_activations(cfg, seed=0)
+    w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=0)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    a = pkg.MoeFfnW8A8(w13, w13s, w2, w2s).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
+    b = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, weight_nz=True).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))

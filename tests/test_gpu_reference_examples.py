@@ -4,12 +4,14 @@ libcust_opapi.so (recipe: `make -C oracle ref_examples`, binaries in oracle/_ref
   moe/moe_init_routing_v2/examples/test_aclnn_moe_init_routing_v2.cpp        drop/pad routing of 3 tokens, E=3, C=2
   moe/moe_finalize_routing_v2/examples/test_aclnn_moe_finalize_routing_v2.cpp fp32 finalize with x1, x2, bias
   moe/moe_gating_top_k_softmax_v2/examples/test_aclnn_moe_gating_top_k_softmax_v2.cpp   softmax then top-2 of 3x4 logits
+  gmm/grouped_matmul_swiglu_quant/examples/test_aclnn_grouped_matmul_swiglu_quant.cpp   FRACTAL_NZ weight [4, 128, 448, 16, 32],
+                                                                              8192 x 7168 rows, all inputs zero
   gmm/grouped_matmul/examples/test_aclnn_grouped_matmul.cpp                   fp16 grouped matmul via V5
-  gmm/grouped_matmul_swiglu_quant/examples/test_aclnn_grouped_matmul_swiglu_quant.cpp   FRACTAL_NZ weight
   moe/moe_init_routing_v3/examples/test_aclnn_moe_init_routing_v3.cpp         FLOAT rows into an INT8 output, quantMode -1
 
-The first three must print what the oracle computes from the same literals (held below as data).  The last three use a
-data type / weight format / dtype pairing outside this build's path: they must fail cleanly in the first phase with
+The first three must print what the oracle computes from the same literals (held below as data); the SwiGLU example
+must run through (its group list is all zero, so no row belongs to a group and the outputs keep their zeros).  The
+last two use a data type / dtype pairing outside this build's path: they must fail cleanly in the first phase with
 ACLNN_ERR_PARAM_INVALID (161002), the reference's code for an unsupported combination, not crash.
 """
 import os
@@ -76,10 +78,27 @@ def test_gating_example(oracle, dev):
     np.testing.assert_allclose(got, want.reshape(-1), rtol=0, atol=1e-6)   # six printed decimals
 
 
+def test_swiglu_example_with_nz_weight(dev, tmp_path):
+    """Prints 16.8 million result lines: they go to a file and only its two ends are read."""
+    path = os.path.join(EXAMPLES, "test_aclnn_grouped_matmul_swiglu_quant")
+    if not os.path.exists(path):
+        pytest.skip("the example is not built (needs the reference sources: make -C oracle ref_examples)")
+    log = tmp_path / "swiglu_example.txt"
+    with open(log, "wb") as f:
+        rc = subprocess.run([path], stdout=f, stderr=subprocess.STDOUT, timeout=110).returncode
+    size = os.path.getsize(log)
+    with open(log, "rb") as f:
+        head = f.read(4096).decode(errors="replace")
+        f.seek(max(0, size - 4096))
+        tail = f.read().decode(errors="replace")
+    assert rc == 0, head + " ... " + tail
+    assert "ERROR" not in head and "ERROR" not in tail
+    assert head.startswith("result[0] is: 0\n") or "result[0] is: 0\n" in head
+    assert tail.rstrip().endswith("result[8191] is: 0.000000")      # the last per-row output scale
+
+
 @pytest.mark.parametrize("name,api", [("test_aclnn_grouped_matmul", "aclnnGroupedMatmulV5GetWorkspaceSize"),
-                                      ("test_aclnn_moe_init_routing_v3", "aclnnMoeInitRoutingV3GetWorkspaceSize"),
-                                      ("test_aclnn_grouped_matmul_swiglu_quant",
-                                       "aclnnGroupedMatmulSwigluQuantGetWorkspaceSize")])
+                                      ("test_aclnn_moe_init_routing_v3", "aclnnMoeInitRoutingV3GetWorkspaceSize")])
 def test_unsupported_examples_fail_cleanly(name, api, dev):
     rc, text = _run(name)
     assert "%s failed. ERROR: 161002" % api in text, text
