@@ -2,7 +2,9 @@
  * CPU oracle for the quantized MoE expert-FFN path.  TEST INFRASTRUCTURE ONLY.
  *
  * A plain-C restatement (OpenMP over rows) of the numerics of the four reference operators on the path:
- *   MoeInitRoutingV2 -> GroupedMatmulSwigluQuant -> GroupedMatmul (int8 down projection) -> MoeFinalizeRoutingV2.
+ *   MoeInitRoutingV2 -> GroupedMatmulSwigluQuant -> GroupedMatmul (int8 down projection) -> MoeFinalizeRoutingV2,
+ * and of the operators around it that the library also provides: MoeGatingTopKSoftmaxV2, MoeInitRoutingV3 (with and
+ * without dynamic quantisation) and GroupedMatmulFinalizeRouting.
  * It exists to check the HIP kernels and to be timed as the CPU baseline.  Nothing in the shipped library links,
  * loads or calls it; only the test-suite, the smoke check and the benchmark's cpu_baseline leg may.
  *
@@ -22,6 +24,14 @@
  *   finalize       : numpy fp32 closed form; example literal
  *                    (moe/moe_finalize_routing_v2/examples/test_aclnn_moe_finalize_routing_v2.cpp:102-110);
  *                    column/row arrangement equivalence; the reference generator's shapes.
+ *   gating         : float64 numpy softmax + stable descending argsort; closed form of the example's input
+ *                    (moe/moe_gating_top_k_softmax_v2/examples/test_aclnn_moe_gating_top_k_softmax_v2.cpp:93); the
+ *                    ties-away narrowing against every half-precision midpoint.
+ *                    PARITY UNPINNED at the last-ulp level and in the order among equal values: SoftMax, TopK and
+ *                    Sort32 live in the CANN library and the reference holds no numbers for this operator.
+ *   routing V3     : numpy stable argsort of the in-range positions; equality with the V2 function on the whole
+ *                    range; dynamic quantisation against a numpy restatement bit for bit.
+ *   fused combine  : float64 numpy (exact matmul per group + np.add.at); equality with "dequantise, then scatter".
  */
 #include <math.h>
 #include <stdint.h>
