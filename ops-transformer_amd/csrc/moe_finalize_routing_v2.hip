@@ -85,7 +85,9 @@ __global__ __launch_bounds__(256) void FinalizeKernel(FinalizeArgs a, int scaleI
     const bool skipsAllowed = a.dropPadMode == 1 || a.dropPadMode == 3;
     constexpr int dataIsF16 = Codec::kRoundEveryOp ? 1 : 0;
 
-    for (int64_t pk = lane; pk < packets; pk += kLanesPerToken) {
+    // gridDim.y workgroups share a token's row: slice y takes packets y * lanes + lane, + lanes * gridDim.y, ...
+    for (int64_t pk = lane + static_cast<int64_t>(blockIdx.y) * kLanesPerToken; pk < packets;
+         pk += static_cast<int64_t>(kLanesPerToken) * gridDim.y) {
         float acc[kVec];
         bool init = false;
         if (a.x1 != nullptr) {
@@ -156,8 +158,10 @@ class FinalizeExecutor : public aclOpExecutor {
             const unsigned blocks = static_cast<unsigned>((args.tokens + 3) / 4);
             hipLaunchKernelGGL((FinalizeKernel<Codec, kVec, 64>), dim3(blocks), dim3(256), 0, stream, args, scaleIsF32);
         } else {
-            hipLaunchKernelGGL((FinalizeKernel<Codec, kVec, 256>), dim3(static_cast<unsigned>(args.tokens)), dim3(256), 0,
-                               stream, args, scaleIsF32);
+            // one 256-lane slice of the row per workgroup: short rows of work, many of them in flight
+            const unsigned slices = static_cast<unsigned>((packets + 255) / 256);
+            hipLaunchKernelGGL((FinalizeKernel<Codec, kVec, 256>), dim3(static_cast<unsigned>(args.tokens), slices), dim3(256),
+                               0, stream, args, scaleIsF32);
         }
     }
 
