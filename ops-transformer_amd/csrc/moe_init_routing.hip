@@ -102,6 +102,8 @@ struct CountOutputs {
     int32_t* beforeCapacity;  // [expertNum] or nullptr
     int32_t flag;             // 1 cumsum, 2 count (applies to countOrCumsum)
     int32_t expertNum;
+    int64_t* wide;            // [expertNum] or nullptr: the same counts as int64 (V3), cumsum when wideCumsum
+    int32_t wideCumsum;
 };
 
 // One workgroup of 1024 threads.  With B bins, 1024 / B threads share each digit value (one thread owns two values when
@@ -155,6 +157,7 @@ __global__ __launch_bounds__(1024) void DigitScanKernel(SortPass p, CountOutputs
             if (b < co.expertNum) {
                 if (co.countOrCumsum != nullptr) co.countOrCumsum[b] = co.flag == 1 ? base + total[j] : total[j];
                 if (co.beforeCapacity != nullptr) co.beforeCapacity[b] = total[j];
+                if (co.wide != nullptr) co.wide[b] = co.wideCumsum ? base + total[j] : total[j];
             }
             base += total[j];
         }
@@ -567,6 +570,10 @@ class InitRoutingExecutor : public aclOpExecutor {
         workspaceBytes = total > 0 ? off : 0;
     }
 
+    // V3 counts or cumsum over the whole expert range come straight out of the scan kernel (one launch fewer);
+    // key/value pairs and a proper sub-range (whose sentinel bin must not be counted) go through CountV3Kernel.
+    bool WideCountsFromScan() const { return v3 && !remap && countMode != 2 && passes == 1; }
+
     template <typename Vec>
     void LaunchGather(char* ws, hipStream_t stream) const {
         if (dropPad) {
@@ -621,10 +628,14 @@ class InitRoutingExecutor : public aclOpExecutor {
             p.shift = shift;
             p.bits = bitsPerPass[pass];
             p.flipSign = (signedRange && last) ? 1 : 0;
-            CountOutputs co{nullptr, nullptr, countFlag, static_cast<int32_t>(expertNum)};
+            CountOutputs co{nullptr, nullptr, countFlag, static_cast<int32_t>(expertNum), nullptr, 0};
             if (last && passes == 1) {
                 co.countOrCumsum = countOrCumsum;
                 co.beforeCapacity = beforeCapacity;
+                if (WideCountsFromScan()) {
+                    co.wide = count64;
+                    co.wideCumsum = countMode == 0 ? 1 : 0;
+                }
             }
             InverseMap im{last ? expandedRowIdx : nullptr, dropPad, static_cast<int32_t>(capacity),
                           last ? gatherIdxOut : nullptr, (remap && passes == 1) ? expertEnd - expertStart : -1};
@@ -645,13 +656,15 @@ class InitRoutingExecutor : public aclOpExecutor {
             shift += bitsPerPass[pass];
         }
         if (passes > 1 && (countOrCumsum != nullptr || beforeCapacity != nullptr)) {
-            CountOutputs co{countOrCumsum, beforeCapacity, countFlag, static_cast<int32_t>(expertNum)};
+            CountOutputs co{countOrCumsum, beforeCapacity, countFlag, static_cast<int32_t>(expertNum), nullptr, 0};
             const unsigned blocks = static_cast<unsigned>((expertNum + 255) / 256);
             hipLaunchKernelGGL(CountFromSortedKernel, dim3(blocks), dim3(256), 0, stream, keysIn, total, co);
         }
-        if (v3) {
+        if (v3 && !WideCountsFromScan()) {
             CountV3Args ca{countOrCumsum, count64, expertEnd - expertStart, expertStart, countMode, kvPairs};
             hipLaunchKernelGGL(CountV3Kernel, dim3(1), dim3(1024), 0, stream, ca);
+        }
+        if (v3) {
             if (scale != nullptr && !dynamicQuant && !(rowBytes > 0 && tokens > 0)) {  // otherwise the row gather carries the scales
                 hipLaunchKernelGGL(ScatterScaleKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
                                    stream, scale, expandedScale, expandedRowIdx, total, static_cast<int32_t>(topK));
