@@ -56,6 +56,8 @@ _VPP = ctypes.POINTER(ctypes.c_void_p)
 _PHASE1_SIGNATURES = {
     "aclnnMoeInitRoutingV2GetWorkspaceSize":
         [_VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _VP, _VP, _VP, _VP, _U64P, _VPP],
+    "aclnnMoeInitRoutingQuantV2GetWorkspaceSize":
+        [_VP, _VP, _VP, _VP, _I64, _I64, _I64, _I64, _I64, ctypes.c_bool, _I64, _VP, _VP, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize":
         [_VP, _VP, _I64, _I64, ctypes.c_bool, _VP, _VP, _VP, _U64P, _VPP],
     "aclnnMoeInitRoutingV3GetWorkspaceSize":
@@ -83,7 +85,7 @@ _PHASE1_SIGNATURES = {
     "aclnnMoeFinalizeRoutingV2GetWorkspaceSize":
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _U64P, _VPP],
 }
-_PHASE2 = ["aclnnGroupedMatmulSwigluQuantWeightNZ", "aclnnGroupedMatmulWeightNz",
+_PHASE2 = ["aclnnMoeInitRoutingQuantV2", "aclnnGroupedMatmulSwigluQuantWeightNZ", "aclnnGroupedMatmulWeightNz",
            "aclnnGroupedMatmulFinalizeRoutingWeightNz", "aclnnGroupedMatmulFinalizeRoutingWeightNzV2", "aclnnGroupedMatmulFinalizeRouting", "aclnnGroupedMatmulFinalizeRoutingV2", "aclnnGroupedMatmulFinalizeRoutingV3",
            "aclnnMoeGatingTopKSoftmaxV2", "aclnnMoeInitRoutingV2", "aclnnMoeInitRoutingV3", "aclnnGroupedMatmulSwigluQuant", "aclnnGroupedMatmulV4", "aclnnGroupedMatmulV5",
            "aclnnMoeFinalizeRoutingV2"]
@@ -282,6 +284,37 @@ def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_n
     finally:
         h.close()
     return expanded_x, expanded_row_idx, count_out, before_out
+
+
+def moe_init_routing_quant_v2(x, expert_idx, quant_mode, scale=None, offset=None, active_num=0, expert_capacity=0,
+                              expert_num=0, drop_pad_mode=0, expert_tokens_count_or_cumsum_flag=0,
+                              expert_tokens_before_capacity_flag=False, workspace=None):
+    """aclnnMoeInitRoutingQuantV2.  Returns (expandedX int8, expandedRowIdx, countOrCumsum | None, beforeCapacity | None,
+    dynamicQuantScale | None)."""
+    T, H = x.shape
+    K = expert_idx.shape[1]
+    dev = x.device
+    if drop_pad_mode == 1:
+        expanded_x = torch.zeros((expert_num, expert_capacity, H), dtype=torch.int8, device=dev)
+        rows = expert_num * expert_capacity
+        count_flag, before_flag = 0, expert_tokens_before_capacity_flag
+    else:
+        rows = T * K if active_num == 0 else min(T * K, active_num)
+        expanded_x = torch.zeros((rows, H), dtype=torch.int8, device=dev)
+        count_flag, before_flag = expert_tokens_count_or_cumsum_flag, False
+    row_idx = torch.empty((T * K,), dtype=torch.int32, device=dev)
+    counts = torch.zeros((expert_num,), dtype=torch.int32, device=dev) if count_flag else None
+    before = torch.zeros((expert_num,), dtype=torch.int32, device=dev) if before_flag else None
+    dyn = torch.zeros((rows,), dtype=torch.float32, device=dev) if quant_mode == 1 else None
+    h = _Handles()
+    try:
+        args = [h.tensor(x), h.tensor(expert_idx), h.tensor(scale), h.tensor(offset), active_num, expert_capacity,
+                expert_num, drop_pad_mode, expert_tokens_count_or_cumsum_flag, expert_tokens_before_capacity_flag,
+                quant_mode, h.tensor(expanded_x), h.tensor(row_idx), h.tensor(counts), h.tensor(before), h.tensor(dyn)]
+        _run_two_phase("aclnnMoeInitRoutingQuantV2", args, dev, workspace)
+    finally:
+        h.close()
+    return expanded_x, row_idx, counts, before, dyn
 
 
 def moe_gating_top_k_softmax_v2(x, k, renorm=0, finished=None, output_softmax=False, out=None):

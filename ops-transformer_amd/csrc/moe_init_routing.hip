@@ -24,6 +24,7 @@
 
 #include <hip/hip_fp16.h>
 
+#include "aclnnop/aclnn_moe_init_routing_quant_v2.h"
 #include "aclnnop/aclnn_moe_init_routing_v2.h"
 #include "aclnnop/aclnn_moe_init_routing_v3.h"
 
@@ -375,11 +376,16 @@ struct QuantGatherArgs {
     float* expandedScale;
     const int32_t* expandedRowIdx;  // scatter-type map
     const int32_t* expertIdx;
-    const float* smooth;            // [active, cols] or nullptr
+    const float* smooth;            // [active, cols], [1, cols] or nullptr
     int64_t cols;
+    int64_t limit;                  // destinations at or beyond it are not written
     int32_t topK;
     int32_t expertStart;
     int32_t dtype;                  // ACL_FLOAT, ACL_FLOAT16, ACL_BF16
+    int32_t smoothPerExpert;        // 1: smooth row = expert - expertStart; 0: one row for every expert
+    // static quantisation (MoeInitRoutingQuantV2 quantMode 0): both non-null, one float each; no per-row scale then
+    const float* staticScale;
+    const float* staticOffset;
 };
 
 __device__ __forceinline__ float LoadAsFloat(const void* p, int64_t i, int dtype) {
@@ -418,18 +424,32 @@ __device__ __forceinline__ int8_t QuantizeOne(float v, float scale) {
     return static_cast<int8_t>(static_cast<int>(r));
 }
 
+// Static quantisation of MoeInitRoutingQuantV2 (moe/moe_init_routing_quant_v2/op_kernel/moe_v2_gather_quant.h:93-133): the
+// value is narrowed to half precision, multiplied by half(scale) and increased by half(offset) in half arithmetic (each
+// step rounds to nearest even), then rounded to the nearest integer and saturated to int8.
+__device__ __forceinline__ int8_t StaticQuantOne(float v, __half hScale, __half hOffset) {
+    const __half u = __hadd(__hmul(__float2half_rn(v), hScale), hOffset);
+    const float r = fminf(fmaxf(rintf(__half2float(u)), -128.f), 127.f);
+    return static_cast<int8_t>(static_cast<int>(r));
+}
+
 template <int kVec>
 __global__ __launch_bounds__(kGatherThreads) void QuantGatherRowsKernel(QuantGatherArgs a) {
     __shared__ float waveMax[kGatherThreads / kWaveSize];
     const int64_t n = blockIdx.x;
-    const int copies = a.smooth != nullptr ? a.topK : 1;
+    const bool isStatic = a.staticScale != nullptr;
+    const __half hScale = isStatic ? __float2half_rn(a.staticScale[0]) : __float2half_rn(0.f);
+    const __half hOffset = isStatic ? __float2half_rn(a.staticOffset[0]) : __float2half_rn(0.f);
+    const bool perCopy = a.smooth != nullptr && a.smoothPerExpert != 0;  // every copy of the token is scaled differently
+    const int copies = perCopy ? a.topK : 1;
     for (int j = 0; j < copies; ++j) {
         const int32_t dstOne = a.expandedRowIdx[n * a.topK + j];
-        if (a.smooth != nullptr && dstOne < 0) continue;  // uniform over the workgroup
-        const float* smooth =
-            a.smooth != nullptr ? a.smooth + static_cast<int64_t>(a.expertIdx[n * a.topK + j] - a.expertStart) * a.cols : nullptr;
+        if (perCopy && (dstOne < 0 || dstOne >= a.limit)) continue;  // uniform over the workgroup
+        const float* smooth = a.smooth == nullptr ? nullptr
+                              : perCopy ? a.smooth + static_cast<int64_t>(a.expertIdx[n * a.topK + j] - a.expertStart) * a.cols
+                                        : a.smooth;
         float mx = 0.f;
-        for (int64_t c = static_cast<int64_t>(threadIdx.x) * kVec; c < a.cols; c += kGatherThreads * kVec) {
+        for (int64_t c = static_cast<int64_t>(threadIdx.x) * kVec; c < a.cols && !isStatic; c += kGatherThreads * kVec) {
             float v[kVec];
             LoadRowChunk<kVec>(a.x, n * a.cols + c, a.dtype, v);
 #pragma unroll
@@ -446,9 +466,9 @@ __global__ __launch_bounds__(kGatherThreads) void QuantGatherRowsKernel(QuantGat
         for (int w = 1; w < kGatherThreads / kWaveSize; ++w) mx = fmaxf(mx, waveMax[w]);
         const float scale = mx / 127.0f;
 
-        for (int jj = (a.smooth != nullptr ? j : 0); jj < (a.smooth != nullptr ? j + 1 : a.topK); ++jj) {
+        for (int jj = (perCopy ? j : 0); jj < (perCopy ? j + 1 : a.topK) && !isStatic; ++jj) {
             const int32_t dst = a.expandedRowIdx[n * a.topK + jj];
-            if (dst >= 0 && threadIdx.x == 0) a.expandedScale[dst] = scale;
+            if (dst >= 0 && dst < a.limit && threadIdx.x == 0) a.expandedScale[dst] = scale;
         }
         for (int64_t c = static_cast<int64_t>(threadIdx.x) * kVec; c < a.cols; c += kGatherThreads * kVec) {
             int8_t q[kVec];
@@ -457,11 +477,12 @@ __global__ __launch_bounds__(kGatherThreads) void QuantGatherRowsKernel(QuantGat
 #pragma unroll
             for (int i = 0; i < kVec; ++i) {
                 if (smooth != nullptr) v[i] = v[i] * smooth[c + i];
-                q[i] = mx == 0.f ? static_cast<int8_t>(0) : QuantizeOne(v[i], scale);
+                q[i] = isStatic ? StaticQuantOne(v[i], hScale, hOffset)
+                                : (mx == 0.f ? static_cast<int8_t>(0) : QuantizeOne(v[i], scale));
             }
-            for (int jj = (a.smooth != nullptr ? j : 0); jj < (a.smooth != nullptr ? j + 1 : a.topK); ++jj) {
+            for (int jj = (perCopy ? j : 0); jj < (perCopy ? j + 1 : a.topK); ++jj) {
                 const int64_t dst = a.expandedRowIdx[n * a.topK + jj];
-                if (dst < 0) continue;
+                if (dst < 0 || dst >= a.limit) continue;
                 int8_t* out = a.expandedX + dst * a.cols + c;
                 if constexpr (kVec == 4) {
                     *reinterpret_cast<uint32_t*>(out) = static_cast<uint32_t>(static_cast<uint8_t>(q[0])) |
@@ -474,6 +495,13 @@ __global__ __launch_bounds__(kGatherThreads) void QuantGatherRowsKernel(QuantGat
             }
         }
     }
+}
+
+// Drop/pad mode with dynamic quantisation: capacity rows beyond an expert's (capped) count get scale 0.
+__global__ void ZeroUnusedScaleKernel(float* expandedScale, const int32_t* binTotal, int32_t capacity, int32_t experts) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= experts * capacity) return;
+    if (i % capacity >= binTotal[i / capacity]) expandedScale[i] = 0.0f;
 }
 
 // V3: expandedScale[destination] = scale[source / K] through the scatter-type map.
@@ -514,6 +542,9 @@ class InitRoutingExecutor : public aclOpExecutor {
     const float* scale = nullptr;
     float* expandedScale = nullptr;
     bool dynamicQuant = false;                // quantMode 1: `scale` is the optional smooth scale [active, cols]
+    bool smoothPerExpert = true;              // false: the smooth scale is one row [1, cols] for every expert
+    const float* staticScale = nullptr;       // MoeInitRoutingQuantV2 quantMode 0: scale[1], offset[1] on the device
+    const float* staticOffset = nullptr;
     int32_t xDtype = ACL_FLOAT;
     int64_t cols = 0;
     uint64_t offRemapKeys = 0, offCounts = 0, offScatterMap = 0;
@@ -670,11 +701,23 @@ class InitRoutingExecutor : public aclOpExecutor {
                                    stream, scale, expandedScale, expandedRowIdx, total, static_cast<int32_t>(topK));
             }
         }
-        if (dynamicQuant) {
+        if (dynamicQuant || staticScale != nullptr) {
             if (tokens > 0 && cols > 0) {
                 opapi::KernelTimer timer("routing_quant_gather", stream);
-                QuantGatherArgs q{x, reinterpret_cast<int8_t*>(expandedX), expandedScale, expandedRowIdx, expertIdx, scale,
-                                  cols, static_cast<int32_t>(topK), expertStart, xDtype};
+                if (dropPad) {
+                    const int32_t* binTotal = reinterpret_cast<const int32_t*>(ws + offBinTotal);
+                    hipLaunchKernelGGL(ZeroUnusedCapacityKernel<uint8_t>, dim3(static_cast<unsigned>(expertNum * capacity)),
+                                       dim3(kGatherThreads), 0, stream, expandedX, binTotal, static_cast<int32_t>(capacity), cols);
+                    if (dynamicQuant) {
+                        hipLaunchKernelGGL(ZeroUnusedScaleKernel, dim3(static_cast<unsigned>((expertNum * capacity + 255) / 256)),
+                                           dim3(256), 0, stream, expandedScale, binTotal, static_cast<int32_t>(capacity),
+                                           static_cast<int32_t>(expertNum));
+                    }
+                }
+                QuantGatherArgs q{x, reinterpret_cast<int8_t*>(expandedX), expandedScale, expandedRowIdx, expertIdx,
+                                  dynamicQuant ? scale : nullptr, cols, dropPad ? expertNum * capacity : activeRows,
+                                  static_cast<int32_t>(topK), expertStart, xDtype, smoothPerExpert ? 1 : 0, staticScale,
+                                  staticOffset};
                 const bool wide = cols % 4 == 0 && reinterpret_cast<uintptr_t>(expandedX) % 4 == 0 &&
                                   reinterpret_cast<uintptr_t>(x) % 16 == 0;
                 if (wide) hipLaunchKernelGGL(QuantGatherRowsKernel<4>, dim3(static_cast<unsigned>(tokens)), dim3(kGatherThreads), 0, stream, q);
@@ -695,13 +738,15 @@ class InitRoutingExecutor : public aclOpExecutor {
     }
 };
 
-}  // namespace
-
-extern "C" aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
-    const aclTensor* x, const aclTensor* expertIdx, int64_t activeNum, int64_t expertCapacity, int64_t expertNum,
-    int64_t dropPadMode, int64_t expertTokensCountOrCumsumFlag, bool expertTokensBeforeCapacityFlag,
-    const aclTensor* expandedXOut, const aclTensor* expandedRowIdxOut, const aclTensor* expertTokensCountOrCumsumOut,
-    const aclTensor* expertTokensBeforeCapacityOut, uint64_t* workspaceSize, aclOpExecutor** executor) {
+// Shared first phase of aclnnMoeInitRoutingV2 (quantMode -1: rows are copied) and aclnnMoeInitRoutingQuantV2
+// (quantMode 0: static, 1: dynamic quantisation to INT8; rules of
+// moe/moe_init_routing_quant_v2/op_host/moe_init_routing_quant_v2_tiling.cpp:132-219).
+aclnnStatus PlanRoutingV2(const aclTensor* x, const aclTensor* expertIdx, const aclTensor* scaleOptional,
+                          const aclTensor* offsetOptional, int64_t activeNum, int64_t expertCapacity, int64_t expertNum,
+                          int64_t dropPadMode, int64_t expertTokensCountOrCumsumFlag, bool expertTokensBeforeCapacityFlag,
+                          int64_t quantMode, const aclTensor* expandedXOut, const aclTensor* expandedRowIdxOut,
+                          const aclTensor* expertTokensCountOrCumsumOut, const aclTensor* expertTokensBeforeCapacityOut,
+                          const aclTensor* dynamicQuantScaleOut, uint64_t* workspaceSize, aclOpExecutor** executor) {
     using namespace opapi;
     ClearError();
     OPAPI_CHECK_NOTNULL(x, "x");
@@ -715,7 +760,14 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
     OPAPI_CHECK(x->dtype == ACL_FLOAT || x->dtype == ACL_FLOAT16 || x->dtype == ACL_BF16 || x->dtype == ACL_INT8, kInvalid,
                 "x dtype %d is not supported (FLOAT, FLOAT16, BF16, INT8)", (int)x->dtype);
     OPAPI_CHECK(expertIdx->dtype == ACL_INT32, kInvalid, "expertIdx must be INT32");
-    OPAPI_CHECK(expandedXOut->dtype == x->dtype, kInvalid, "expandedXOut dtype must equal x dtype");
+    const bool quant = quantMode >= 0;
+    if (quant) {
+        OPAPI_CHECK(quantMode == 0 || quantMode == 1, kInvalid, "The quantMode should be 0 or 1.");
+        OPAPI_CHECK(x->dtype != ACL_INT8, kInvalid, "quantisation takes FLOAT, FLOAT16 or BF16 rows, not INT8");
+        OPAPI_CHECK(expandedXOut->dtype == ACL_INT8, kInvalid, "expandedXOut must be INT8 when the rows are quantised");
+    } else {
+        OPAPI_CHECK(expandedXOut->dtype == x->dtype, kInvalid, "expandedXOut dtype must equal x dtype");
+    }
     OPAPI_CHECK(expandedRowIdxOut->dtype == ACL_INT32, kInvalid, "expandedRowIdxOut must be INT32");
     OPAPI_CHECK(x->dims.size() == 2, kInvalid, "The dim number of x should be 2.");
     OPAPI_CHECK(expertIdx->dims.size() == 2, kInvalid, "The dim number of expertIdx should be 2.");
@@ -784,9 +836,52 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
         OPAPI_CHECK(cols == 0 || (x->data != nullptr && expandedXOut->data != nullptr), ACLNN_ERR_PARAM_NULLPTR,
                     "x / expandedXOut carry no device memory");
     }
+    bool smoothPerExpert = false;
+    if (quantMode == 0) {
+        OPAPI_CHECK(scaleOptional != nullptr, ACLNN_ERR_PARAM_NULLPTR, "scale is nullptr!");
+        OPAPI_CHECK(offsetOptional != nullptr, ACLNN_ERR_PARAM_NULLPTR, "offset is nullptr!");
+        OPAPI_CHECK(scaleOptional->dtype == ACL_FLOAT, kInvalid, "The data type of scale should be float.");
+        OPAPI_CHECK(offsetOptional->dtype == ACL_FLOAT, kInvalid, "The data type of offset should be float.");
+        OPAPI_CHECK(scaleOptional->dims.size() == 1, kInvalid, "The dim number of scale should be 1.");
+        OPAPI_CHECK(scaleOptional->dims[0] == 1, kInvalid, "The first dim of scale should be 1.");
+        OPAPI_CHECK(offsetOptional->dims.size() == 1, kInvalid, "The dim number of offset should be 1.");
+        OPAPI_CHECK(offsetOptional->dims[0] == 1, kInvalid, "The first dim of offset should be 1.");
+        OPAPI_CHECK(scaleOptional->data != nullptr && offsetOptional->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
+                    "scale / offset carry no device memory");
+    } else if (quantMode == 1) {
+        if (scaleOptional != nullptr) {
+            OPAPI_CHECK(scaleOptional->dtype == ACL_FLOAT, kInvalid, "The data type of scale should be float.");
+            OPAPI_CHECK(scaleOptional->dims.size() == 2, kInvalid, "The dim number of scale should be 2.");
+            OPAPI_CHECK(scaleOptional->dims[0] == 1 || scaleOptional->dims[0] == expertNum, kInvalid,
+                        "The first dim of scale should be 1 or expert_num.");
+            OPAPI_CHECK(scaleOptional->dims[1] == cols, kInvalid, "The second dim of scale should be %lld.", (long long)cols);
+            OPAPI_CHECK(IsContiguous(scaleOptional) && (total == 0 || scaleOptional->data != nullptr), kInvalid,
+                        "scale must be contiguous device memory");
+            smoothPerExpert = scaleOptional->dims[0] != 1;
+        }
+        OPAPI_CHECK(dynamicQuantScaleOut != nullptr, ACLNN_ERR_PARAM_NULLPTR, "DynamicQuantScale is nullptr!");
+        OPAPI_CHECK(dynamicQuantScaleOut->dtype == ACL_FLOAT, kInvalid, "The data type of dynamicQuantScale should be FLOAT.");
+        OPAPI_CHECK(dynamicQuantScaleOut->dims.size() == 1, kInvalid, "The dim number of dynamicQuantScale should be 1.");
+        const int64_t want = dropPadMode == 0 ? activeRows : expertNum * expertCapacity;
+        OPAPI_CHECK(dynamicQuantScaleOut->dims[0] == want, kInvalid, "The first dim of dynamicQuantScale should be %lld.",
+                    (long long)want);
+        OPAPI_CHECK(IsContiguous(dynamicQuantScaleOut) && (total == 0 || dynamicQuantScaleOut->data != nullptr), kInvalid,
+                    "dynamicQuantScale must be contiguous device memory");
+    }
 
     auto* ex = new (std::nothrow) InitRoutingExecutor();
     OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
+    if (quantMode == 0) {
+        ex->staticScale = reinterpret_cast<const float*>(DataPtr(scaleOptional));
+        ex->staticOffset = reinterpret_cast<const float*>(DataPtr(offsetOptional));
+    } else if (quantMode == 1) {
+        ex->dynamicQuant = true;
+        ex->scale = reinterpret_cast<const float*>(DataPtr(scaleOptional));
+        ex->smoothPerExpert = smoothPerExpert;
+        ex->expandedScale = reinterpret_cast<float*>(DataPtr(dynamicQuantScaleOut));
+    }
+    ex->xDtype = x->dtype;
+    ex->cols = cols;
     ex->x = DataPtr(x);
     ex->expertIdx = reinterpret_cast<const int32_t*>(DataPtr(expertIdx));
     ex->expandedX = DataPtr(expandedXOut);
@@ -806,6 +901,42 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
+    const aclTensor* x, const aclTensor* expertIdx, int64_t activeNum, int64_t expertCapacity, int64_t expertNum,
+    int64_t dropPadMode, int64_t expertTokensCountOrCumsumFlag, bool expertTokensBeforeCapacityFlag,
+    const aclTensor* expandedXOut, const aclTensor* expandedRowIdxOut, const aclTensor* expertTokensCountOrCumsumOut,
+    const aclTensor* expertTokensBeforeCapacityOut, uint64_t* workspaceSize, aclOpExecutor** executor) {
+    return PlanRoutingV2(x, expertIdx, nullptr, nullptr, activeNum, expertCapacity, expertNum, dropPadMode,
+                         expertTokensCountOrCumsumFlag, expertTokensBeforeCapacityFlag, /*quantMode=*/-1, expandedXOut,
+                         expandedRowIdxOut, expertTokensCountOrCumsumOut, expertTokensBeforeCapacityOut, nullptr, workspaceSize,
+                         executor);
+}
+
+extern "C" aclnnStatus aclnnMoeInitRoutingQuantV2GetWorkspaceSize(
+    const aclTensor* x, const aclTensor* expertIdx, const aclTensor* scaleOptional, const aclTensor* offsetOptional,
+    int64_t activeNum, int64_t expertCapacity, int64_t expertNum, int64_t dropPadMode,
+    int64_t expertTokensCountOrCumsumFlag, bool expertTokensBeforeCapacityFlag, int64_t quantMode,
+    const aclTensor* expandedXOut, const aclTensor* expandedRowIdxOut, const aclTensor* expertTokensCountOrCumsumOutOptional,
+    const aclTensor* expertTokensBeforeCapacityOutOptional, const aclTensor* dynamicQuantScaleOutOptional,
+    uint64_t* workspaceSize, aclOpExecutor** executor) {
+    if (quantMode < 0 || quantMode > 1) {
+        opapi::ClearError();
+        opapi::SetError("The quantMode should be 0 or 1.");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    return PlanRoutingV2(x, expertIdx, scaleOptional, offsetOptional, activeNum, expertCapacity, expertNum, dropPadMode,
+                         expertTokensCountOrCumsumFlag, expertTokensBeforeCapacityFlag, quantMode, expandedXOut,
+                         expandedRowIdxOut, expertTokensCountOrCumsumOutOptional, expertTokensBeforeCapacityOutOptional,
+                         dynamicQuantScaleOutOptional, workspaceSize, executor);
+}
+
+extern "C" aclnnStatus aclnnMoeInitRoutingQuantV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
+                                                  aclrtStream stream) {
+    return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
 }
 
 extern "C" aclnnStatus aclnnMoeInitRoutingV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,

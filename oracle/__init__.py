@@ -212,6 +212,40 @@ def moe_init_routing_v3_quant(x, expert_idx, smooth=None, expert_num=0, expert_r
     return ex, out_idx, counts, ex_scale
 
 
+def moe_init_routing_quant_v2(x, expert_idx, quant_mode, scale=None, offset=None, active_num=0, expert_capacity=0,
+                              expert_num=0, drop_pad_mode=0, count_flag=0, before_capacity_flag=False, dtype=DT_F32):
+    """MoeInitRoutingQuantV2.  x: fp32, or uint16 bit patterns for DT_F16 / DT_BF16.  quant_mode 0: scale, offset are
+    one float each; 1: scale is None or a smooth scale [1 or expert_num, cols].
+    Returns (expandedX int8, expandedRowIdx, countOrCumsum | None, beforeCapacity | None, dynamicQuantScale | None)."""
+    x = _c(x)
+    T, cols = x.shape
+    idx = _c(expert_idx, np.int32)
+    K = idx.shape[1]
+    M = T * K
+    if drop_pad_mode == 1:
+        ex = np.zeros((expert_num, expert_capacity, cols), np.int8)
+        rows = expert_num * expert_capacity
+        count_flag = 0
+    else:
+        rows = M if active_num == 0 else min(M, active_num)
+        ex = np.zeros((rows, cols), np.int8)
+        before_capacity_flag = False
+    ri = np.zeros((M,), np.int32)
+    cnt = np.zeros((expert_num,), np.int32) if count_flag else None
+    bef = np.zeros((expert_num,), np.int32) if before_capacity_flag else None
+    dyn = np.zeros((rows,), np.float32) if quant_mode == 1 else None
+    sc = None if scale is None else _c(np.atleast_1d(scale), np.float32)
+    of = None if offset is None else _c(np.atleast_1d(offset), np.float32)
+    smooth_rows = 1 if (sc is None or quant_mode == 0) else sc.shape[0]
+    rc = lib().oracle_moe_init_routing_quant_v2(
+        _p(x), ctypes.c_int(dtype), ctypes.c_int64(cols), _p(idx), ctypes.c_int64(T), ctypes.c_int64(K),
+        ctypes.c_int64(active_num), ctypes.c_int64(expert_capacity), ctypes.c_int64(expert_num),
+        ctypes.c_int64(drop_pad_mode), ctypes.c_int64(count_flag), ctypes.c_int(int(before_capacity_flag)),
+        ctypes.c_int64(quant_mode), _p(sc), _p(of), ctypes.c_int64(smooth_rows), _p(ex), _p(ri), _p(cnt), _p(bef), _p(dyn))
+    assert rc == 0
+    return ex, ri, cnt, bef, dyn
+
+
 # ----------------------------------------------------------------------------------------------- GEMMs
 def _gemm_common(x, w, w_trans, group_list, rows):
     x = _c(x, np.int8)

@@ -4,7 +4,7 @@
  * A plain-C restatement (OpenMP over rows) of the numerics of the four reference operators on the path:
  *   MoeInitRoutingV2 -> GroupedMatmulSwigluQuant -> GroupedMatmul (int8 down projection) -> MoeFinalizeRoutingV2,
  * and of the operators around it that the library also provides: MoeGatingTopKSoftmaxV2, MoeInitRoutingV3 (with and
- * without dynamic quantisation) and GroupedMatmulFinalizeRouting.
+ * without dynamic quantisation), MoeInitRoutingQuantV2 and GroupedMatmulFinalizeRouting.
  * It exists to check the HIP kernels and to be timed as the CPU baseline.  Nothing in the shipped library links,
  * loads or calls it; only the test-suite, the smoke check and the benchmark's cpu_baseline leg may.
  *
@@ -31,6 +31,9 @@
  *                    Sort32 live in the CANN library and the reference holds no numbers for this operator.
  *   routing V3     : numpy stable argsort of the in-range positions; equality with the V2 function on the whole
  *                    range; dynamic quantisation against a numpy restatement bit for bit.
+ *   routing QuantV2: static mode against numpy float16 arithmetic bit for bit (saturation and ties included); dynamic
+ *                    mode against the V3 function on the whole range; the example's literals
+ *                    (moe/moe_init_routing_quant_v2/examples/test_aclnn_moe_init_routing_quant_v2.cpp:71-108).
  *   fused combine  : float64 numpy (exact matmul per group + np.add.at); equality with "dequantise, then scatter".
  */
 #include <math.h>
@@ -377,6 +380,68 @@ ORACLE_API int oracle_moe_init_routing_v3_quant(const void* x, int dtype, int64_
 
 ORACLE_API void oracle_f32_to_f16_trunc_value(const float* in, float* out, int64_t n) {
     for (int64_t i = 0; i < n; i++) out[i] = f32_to_f16_trunc_value(in[i]);
+}
+
+/* MoeInitRoutingQuantV2: the routing of oracle_moe_init_routing_v2 with the gathered rows quantised to int8.
+ *   quantMode 0 (static, moe/moe_init_routing_quant_v2/op_kernel/moe_v2_gather_quant.h:93-133): every step in half
+ *     precision, each rounding to nearest even: h = half(x); h = h * half(scale); h = h + half(offset);
+ *     y = int8(rint(h)), saturated.  (A half product or sum formed in fp32 and rounded to half once more equals the
+ *     directly rounded half result: fp32 carries 24 >= 2 * 11 + 2 significand bits.)
+ *   quantMode 1 (dynamic, op_kernel/moe_v2_gather_dynamic_quant.h:120-155): as oracle_moe_init_routing_v3_quant;
+ *     smooth is [smoothRows, cols] with smoothRows 1 (one row for all experts) or expertNum.
+ * Drop/pad mode: unused capacity rows are zero with scale 0.  Rows at or beyond activeRows are not written. */
+ORACLE_API int oracle_moe_init_routing_quant_v2(const void* x, int dtype, int64_t cols, const int32_t* expertIdx, int64_t T,
+                                                int64_t K, int64_t activeNum, int64_t capacity, int64_t expertNum,
+                                                int64_t dropPadMode, int64_t countFlag, int beforeCapacityFlag,
+                                                int64_t quantMode, const float* scale, const float* offset,
+                                                int64_t smoothRows, int8_t* expandedX, int32_t* expandedRowIdx,
+                                                int32_t* countOrCumsum, int32_t* beforeCapacity, float* dynScale) {
+    const int64_t M = T * K;
+    const int rc = oracle_moe_init_routing_v2(NULL, 0, expertIdx, T, K, activeNum, capacity, expertNum, dropPadMode, countFlag,
+                                              beforeCapacityFlag, NULL, expandedRowIdx, countOrCumsum, beforeCapacity);
+    if (rc != 0) return rc;
+    const int64_t limit = dropPadMode == 1 ? expertNum * capacity : (activeNum == 0 ? M : (activeNum < M ? activeNum : M));
+    if (dropPadMode == 1) {
+        memset(expandedX, 0, (size_t)(limit * cols));
+        if (quantMode == 1) for (int64_t d = 0; d < limit; d++) dynScale[d] = 0.f;
+    }
+    const float hs = quantMode == 0 ? f16_to_f32(f32_to_f16(scale[0])) : 0.f;
+    const float ho = quantMode == 0 ? f16_to_f32(f32_to_f16(offset[0])) : 0.f;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; i++) {
+        const int64_t d = expandedRowIdx[i];
+        if (d < 0 || d >= limit) continue;
+        const void* row = x;
+        const int64_t base = (i / K) * cols;
+        if (quantMode == 0) {
+            for (int64_t c = 0; c < cols; c++) {
+                float h = f16_to_f32(f32_to_f16(load_as_f32(row, base + c, dtype)));
+                h = f16_to_f32(f32_to_f16(h * hs));
+                h = f16_to_f32(f32_to_f16(h + ho));
+                float r = rintf(h);
+                r = r > 127.f ? 127.f : (r < -128.f ? -128.f : r);
+                expandedX[d * cols + c] = (int8_t)r;
+            }
+            continue;
+        }
+        const float* sm = scale ? scale + (smoothRows == 1 ? 0 : (int64_t)expertIdx[i] * cols) : NULL;
+        float mx = 0.f;
+        for (int64_t c = 0; c < cols; c++) {
+            float v = load_as_f32(row, base + c, dtype);
+            if (sm) v = v * sm[c];
+            mx = fabsf(v) > mx ? fabsf(v) : mx;
+        }
+        const float s = mx / 127.0f;
+        dynScale[d] = s;
+        for (int64_t c = 0; c < cols; c++) {
+            float v = load_as_f32(row, base + c, dtype);
+            if (sm) v = v * sm[c];
+            float r = mx == 0.f ? 0.f : roundf(f32_to_f16_trunc_value(v / s));
+            r = r > 127.f ? 127.f : (r < -128.f ? -128.f : r);
+            expandedX[d * cols + c] = (int8_t)r;
+        }
+    }
+    return 0;
 }
 
 /* ------------------------------------------------------------------------------------------------ grouped GEMM */

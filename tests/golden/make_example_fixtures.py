@@ -8,9 +8,11 @@ The reference holds no expected numbers for these operators: its examples print 
 tests only run the kernels or compare against generators that need absent packages.  What it does hold is inputs:
   moe/moe_init_routing_v2/examples/test_aclnn_moe_init_routing_v2.cpp:71-96          (drop/pad routing, E=3, C=2)
   moe/moe_init_routing_v3/examples/test_aclnn_moe_init_routing_v3.cpp:123-125        (range [0, 4), counts)
+  moe/moe_init_routing_quant_v2/examples/test_aclnn_moe_init_routing_quant_v2.cpp:71-108 (the V2 case, static quantisation)
   moe/moe_finalize_routing_v2/examples/test_aclnn_moe_finalize_routing_v2.cpp:102-110 (fp32, x1 = x2, bias, mode 0)
   moe/moe_gating_top_k_softmax_v2/examples/test_aclnn_moe_gating_top_k_softmax_v2.cpp:93 (softmax then top-2)
-Definitions used: moe/moe_init_routing_v2/README.md, moe/moe_init_routing_v3/README.md:12-66,
+Definitions used: moe/moe_init_routing_v2/README.md, moe/moe_init_routing_quant_v2/README.md (half-precision
+x * scale + offset, rounded to int8), moe/moe_init_routing_v3/README.md:12-66,
 moe/moe_finalize_routing_v2/README.md, moe/moe_gating_top_k_softmax_v2/README.md:12-30.
 """
 import json
@@ -38,6 +40,21 @@ def routing_v2_drop_pad():
     return {"x": x.tolist(), "expert_idx": idx.tolist(), "expert_num": E, "expert_capacity": C, "drop_pad_mode": 1,
             "expanded_row_idx": row_idx.tolist(), "expanded_x": expanded.tolist(),
             "expert_tokens_before_capacity": np.bincount(flat, minlength=E).tolist()}
+
+
+def routing_quant_v2_static():
+    g = routing_v2_drop_pad()
+    scale, offset = np.float32(0.3452), np.float32(1.8369)
+    rows = np.array(g["expanded_x"], np.float32)
+    filled = np.zeros(rows.shape[:2], bool)
+    for dst in g["expanded_row_idx"]:
+        if dst >= 0:
+            filled[dst // g["expert_capacity"], dst % g["expert_capacity"]] = True
+    h = rows.astype(np.float16) * np.float16(scale) + np.float16(offset)          # numpy rounds each half operation
+    q = np.clip(np.rint(h.astype(np.float32)), -128, 127).astype(np.int8)
+    q[~filled] = 0
+    g.update({"quant_mode": 0, "scale": float(scale), "offset": float(offset), "expanded_x": q.tolist()})
+    return g
 
 
 def routing_v3_counts():
@@ -87,6 +104,7 @@ def gating_softmax_topk():
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
     data = {"moe_init_routing_v2_example": routing_v2_drop_pad(), "moe_init_routing_v3_example": routing_v3_counts(),
+            "moe_init_routing_quant_v2_example": routing_quant_v2_static(),
             "moe_finalize_routing_v2_example": finalize_v2(), "moe_gating_top_k_softmax_v2_example": gating_softmax_topk()}
     with open(os.path.join(here, "reference_examples.json"), "w") as f:
         json.dump(data, f, indent=1)

@@ -31,6 +31,7 @@ def test_headers_declare_the_expected_entry_points():
     names = _declared_symbols()
     for required in ["aclnnMoeInitRoutingV2GetWorkspaceSize", "aclnnMoeInitRoutingV2",
                      "aclnnMoeInitRoutingV3GetWorkspaceSize", "aclnnMoeInitRoutingV3",
+                     "aclnnMoeInitRoutingQuantV2GetWorkspaceSize", "aclnnMoeInitRoutingQuantV2",
                      "aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize", "aclnnMoeGatingTopKSoftmaxV2",
                      "aclnnGroupedMatmulFinalizeRoutingGetWorkspaceSize", "aclnnGroupedMatmulFinalizeRouting",
                      "aclnnGroupedMatmulFinalizeRoutingV2GetWorkspaceSize", "aclnnGroupedMatmulFinalizeRoutingV2",
@@ -187,6 +188,85 @@ def test_gating_nulls(aclnn):
         assert _status(aclnn, "aclnnMoeGatingTopKSoftmaxV2", args)[0] == NULLPTR, pos
     args = _gating_args(aclnn, flag=True, with_sm=False)       # softmax output requested, no tensor for it
     assert _status(aclnn, "aclnnMoeGatingTopKSoftmaxV2", args)[0] == NULLPTR
+
+
+# ------------------------------------------------------------------------------------------------ routing QuantV2
+def _routing_quant_v2_args(aclnn, T_=8, K=2, H=16, E=4, mode=0, C=0, flag=0, before=False, active=0, x_dtype=BF16, quant=0,
+                           with_scale=True, with_offset=True, with_dyn=None, **over):
+    x = T(aclnn, (T_, H), x_dtype)
+    idx = T(aclnn, (T_, K), I32)
+    if quant == 0:
+        scale = T(aclnn, over.get("scale_shape", (1,)), over.get("scale_dtype", F32)) if with_scale else None
+        offset = T(aclnn, over.get("offset_shape", (1,)), over.get("offset_dtype", F32)) if with_offset else None
+    else:
+        scale = T(aclnn, over.get("scale_shape", (E, H)), over.get("scale_dtype", F32)) if with_scale else None
+        offset = None
+    rows = E * C if mode == 1 else (T_ * K if active == 0 else min(T_ * K, active))
+    ex = T(aclnn, over.get("ex_shape", (E, C, H) if mode == 1 else (rows, H)), over.get("ex_dtype", I8))
+    ri = T(aclnn, (T_ * K,), I32)
+    cnt = T(aclnn, (E,), I32) if flag > 0 else None
+    bef = T(aclnn, (E,), I32) if before else None
+    dyn = None
+    if with_dyn if with_dyn is not None else quant == 1:
+        dyn = T(aclnn, over.get("dyn_shape", (rows,)), over.get("dyn_dtype", F32))
+    return [x.h, idx.h, scale.h if scale else None, offset.h if offset else None, active, C, E, mode, flag, before, quant,
+            ex.h, ri.h, cnt.h if cnt else None, bef.h if bef else None, dyn.h if dyn else None]
+
+
+def test_routing_quant_v2_valid(aclnn):
+    for kw in [dict(), dict(x_dtype=F32, flag=1), dict(x_dtype=F16, flag=2), dict(mode=1, C=3, before=True), dict(active=5),
+               dict(quant=1), dict(quant=1, scale_shape=(1, 16)), dict(quant=1, with_scale=False),
+               dict(quant=1, mode=1, C=3, before=True), dict(quant=1, active=5, flag=1), dict(T_=0), dict(quant=1, T_=0)]:
+        code, ws = _status(aclnn, "aclnnMoeInitRoutingQuantV2", _routing_quant_v2_args(aclnn, **kw))
+        assert code == 0, (kw, ws)
+
+
+@pytest.mark.parametrize("kw,fragment", [
+    # rules and messages of moe/moe_init_routing_quant_v2/op_host/moe_init_routing_quant_v2_tiling.cpp:132-219
+    (dict(quant=2), "quantMode should be 0 or 1"),
+    (dict(quant=-1), "quantMode should be 0 or 1"),
+    (dict(x_dtype=I8), "not INT8"),
+    (dict(ex_dtype=BF16), "expandedXOut must be INT8"),
+    (dict(scale_dtype=F16), "data type of scale should be float"),
+    (dict(offset_dtype=F16), "data type of offset should be float"),
+    (dict(scale_shape=(1, 1)), "dim number of scale should be 1"),
+    (dict(scale_shape=(2,)), "first dim of scale should be 1"),
+    (dict(offset_shape=(1, 1)), "dim number of offset should be 1"),
+    (dict(offset_shape=(2,)), "first dim of offset should be 1"),
+    (dict(quant=1, scale_shape=(16,)), "dim number of scale should be 2"),
+    (dict(quant=1, scale_shape=(3, 16)), "first dim of scale should be 1 or expert_num"),
+    (dict(quant=1, scale_shape=(4, 15)), "second dim of scale should be 16"),
+    (dict(quant=1, scale_dtype=F16), "data type of scale should be float"),
+    (dict(quant=1, dyn_shape=(15,)), "first dim of dynamicQuantScale should be 16"),
+    (dict(quant=1, dyn_shape=(16, 1)), "dim number of dynamicQuantScale should be 1"),
+    (dict(quant=1, dyn_dtype=F16), "dynamicQuantScale should be FLOAT"),
+    (dict(quant=1, mode=1, C=3, dyn_shape=(16,)), "first dim of dynamicQuantScale should be 12"),
+    (dict(quant=1, active=5, dyn_shape=(16,)), "first dim of dynamicQuantScale should be 5"),
+    (dict(mode=2), "dropPadMode should be 0 or 1"),
+    (dict(flag=3), "should be 0, 1 or 2"),
+    (dict(mode=1, C=0), "greater than 0 when dropPadMode is 1"),
+    (dict(mode=1, C=9), "cannot be less than expertCapacity"),
+    (dict(ex_shape=(15, 16)), "first dim of expandedX"),
+    (dict(active=-1), "activeNum cannot be less than 0"),
+])
+def test_routing_quant_v2_invalid(aclnn, kw, fragment):
+    code, msg = _status(aclnn, "aclnnMoeInitRoutingQuantV2", _routing_quant_v2_args(aclnn, **kw))
+    assert code == INVALID and fragment in msg, (code, msg)
+
+
+def test_routing_quant_v2_nulls(aclnn):
+    for pos in (0, 1, 11, 12):
+        args = _routing_quant_v2_args(aclnn)
+        args[pos] = None
+        assert _status(aclnn, "aclnnMoeInitRoutingQuantV2", args)[0] == NULLPTR, pos
+    # static quantisation needs both scale and offset (moe_init_routing_quant_v2_tiling.cpp:179-198)
+    assert _status(aclnn, "aclnnMoeInitRoutingQuantV2", _routing_quant_v2_args(aclnn, with_scale=False))[0] == NULLPTR
+    assert _status(aclnn, "aclnnMoeInitRoutingQuantV2", _routing_quant_v2_args(aclnn, with_offset=False))[0] == NULLPTR
+    # dynamic quantisation always emits its scales (moe_init_routing_quant_v2_tiling.cpp:138-140)
+    assert _status(aclnn, "aclnnMoeInitRoutingQuantV2", _routing_quant_v2_args(aclnn, quant=1, with_dyn=False))[0] == NULLPTR
+    args = _routing_quant_v2_args(aclnn, flag=1)
+    args[13] = None
+    assert _status(aclnn, "aclnnMoeInitRoutingQuantV2", args)[0] == NULLPTR
 
 
 # ------------------------------------------------------------------------------------------------ routing V3
@@ -505,7 +585,7 @@ def test_reference_examples_compile_and_link_unmodified():
     assert res.returncode == 0, res.stdout
     for name in ("test_aclnn_moe_init_routing_v2", "test_aclnn_grouped_matmul_swiglu_quant", "test_aclnn_grouped_matmul",
                  "test_aclnn_moe_finalize_routing_v2", "test_aclnn_moe_init_routing_v3",
-                 "test_aclnn_moe_gating_top_k_softmax_v2"):
+                 "test_aclnn_moe_gating_top_k_softmax_v2", "test_aclnn_moe_init_routing_quant_v2"):
         assert os.access(os.path.join(ROOT, "oracle", "_ref", "examples", name), os.X_OK), name
 
 

@@ -31,6 +31,13 @@ def test_oracle_reproduces_the_fixtures(oracle, golden):
     assert ri.tolist() == g["expanded_row_idx"] and cnt.tolist() == g["expert_tokens_count"]
     assert np.array_equal(ex, np.array(g["expanded_x"], np.float32)) and np.array_equal(es, np.array(g["expanded_scale"], np.float32))
 
+    g = golden["moe_init_routing_quant_v2_example"]
+    ex, ri, _, bef, _ = oracle.moe_init_routing_quant_v2(np.array(g["x"], np.float32), np.array(g["expert_idx"], np.int32), 0,
+                                                         g["scale"], g["offset"], expert_capacity=g["expert_capacity"],
+                                                         expert_num=g["expert_num"], drop_pad_mode=1, before_capacity_flag=True)
+    assert ri.tolist() == g["expanded_row_idx"] and bef.tolist() == g["expert_tokens_before_capacity"]
+    assert ex.tolist() == g["expanded_x"]
+
     g = golden["moe_finalize_routing_v2_example"]
     out = oracle.moe_finalize_routing_v2(np.array(g["expanded_x"], np.float32), np.array(g["expanded_row_idx"], np.int32),
                                          np.array(g["x1"], np.float32), np.array(g["x2"], np.float32),
@@ -66,6 +73,13 @@ def test_library_reproduces_the_fixtures(aclnn, golden, dev):
     assert ri.cpu().tolist() == g["expanded_row_idx"] and cnt.cpu().tolist() == g["expert_tokens_count"]
     assert torch.equal(ex.cpu(), torch.tensor(g["expanded_x"], dtype=torch.float32))
     assert torch.equal(es.cpu(), torch.tensor(g["expanded_scale"], dtype=torch.float32))
+
+    g = golden["moe_init_routing_quant_v2_example"]
+    ex, ri, _, bef, _ = aclnn.moe_init_routing_quant_v2(t32(g["x"]), ti(g["expert_idx"]), 0, t32([g["scale"]]), t32([g["offset"]]),
+                                                        expert_capacity=g["expert_capacity"], expert_num=g["expert_num"],
+                                                        drop_pad_mode=1, expert_tokens_before_capacity_flag=True)
+    assert ri.cpu().tolist() == g["expanded_row_idx"] and bef.cpu().tolist() == g["expert_tokens_before_capacity"]
+    assert ex.cpu().tolist() == g["expanded_x"]
 
     g = golden["moe_finalize_routing_v2_example"]
     out = aclnn.moe_finalize_routing_v2(t32(g["expanded_x"]), ti(g["expanded_row_idx"]), x1=t32(g["x1"]), x2=t32(g["x2"]),

@@ -4,12 +4,14 @@ libcust_opapi.so (recipe: `make -C oracle ref_examples`, binaries in oracle/_ref
   moe/moe_init_routing_v2/examples/test_aclnn_moe_init_routing_v2.cpp        drop/pad routing of 3 tokens, E=3, C=2
   moe/moe_finalize_routing_v2/examples/test_aclnn_moe_finalize_routing_v2.cpp fp32 finalize with x1, x2, bias
   moe/moe_gating_top_k_softmax_v2/examples/test_aclnn_moe_gating_top_k_softmax_v2.cpp   softmax then top-2 of 3x4 logits
+  moe/moe_init_routing_quant_v2/examples/test_aclnn_moe_init_routing_quant_v2.cpp       static quantisation (scale 0.3452,
+                                                                              offset 1.8369) of the drop/pad routing above
   gmm/grouped_matmul_swiglu_quant/examples/test_aclnn_grouped_matmul_swiglu_quant.cpp   FRACTAL_NZ weight [4, 128, 448, 16, 32],
                                                                               8192 x 7168 rows, all inputs zero
   gmm/grouped_matmul/examples/test_aclnn_grouped_matmul.cpp                   fp16 grouped matmul via V5
   moe/moe_init_routing_v3/examples/test_aclnn_moe_init_routing_v3.cpp         FLOAT rows into an INT8 output, quantMode -1
 
-The first three must print what the oracle computes from the same literals (held below as data); the SwiGLU example
+The first four must print what the oracle computes from the same literals (held below as data); the SwiGLU example
 must run through (its group list is all zero, so no row belongs to a group and the outputs keep their zeros).  The
 last two use a data type / dtype pairing outside this build's path: they must fail cleanly in the first phase with
 ACLNN_ERR_PARAM_INVALID (161002), the reference's code for an unsupported combination, not crash.
@@ -50,6 +52,19 @@ def test_routing_example(oracle, dev):
     assert _values(text, "expertTokenIdxData", int) == bef.tolist() == [2, 2, 2]
     got = np.array(_values(text, "expandedXData", float), np.float32)
     np.testing.assert_allclose(got, ex.reshape(-1), rtol=0, atol=5e-7)   # printed with six decimals
+
+
+def test_routing_quant_example(oracle, dev):
+    rc, text = _run("test_aclnn_moe_init_routing_quant_v2")
+    assert rc == 0, text
+    x = np.repeat(np.array([[0.1], [0.2], [0.3]], np.float32), 4, axis=1)
+    idx = np.array([[1, 2], [0, 1], [0, 2]], np.int32)
+    ex, ri, _, bef, _ = oracle.moe_init_routing_quant_v2(x, idx, 0, 0.3452, 1.8369, expert_capacity=2, expert_num=3,
+                                                         drop_pad_mode=1, before_capacity_flag=True)
+    assert _values(text, "expandedRowIdxData", int) == ri.tolist() == [2, 4, 0, 3, 1, 5]
+    assert _values(text, "expertTokenIdxData", int) == bef.tolist() == [2, 2, 2]
+    # 0.1 * 0.3452 + 1.8369 ... 0.3 * 0.3452 + 1.8369 all lie in (1.87, 1.95): every slot holds 2
+    assert _values(text, "expandedXData", int) == ex.reshape(-1).tolist() == [2] * 24
 
 
 def test_finalize_example(oracle, dev):

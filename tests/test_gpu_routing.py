@@ -244,3 +244,113 @@ def test_v3_dynamic_quant_feeds_the_gemm(pkg, aclnn, oracle, dev):
                                                    cum.cpu().numpy(), w_trans=True)
     assert np.abs(h.cpu().numpy().astype(np.int32) - h_r.astype(np.int32)).max() <= 1
     np.testing.assert_allclose(hs.cpu().numpy(), hs_r, rtol=1e-2)
+
+
+# ------------------------------------------------------------------------------------------------ QuantV2
+def _quant_v2_inputs(rng, T, K, E, H, dtype_name, oracle, spread=3.0):
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype_name]
+    code = {"f32": oracle.DT_F32, "f16": oracle.DT_F16, "bf16": oracle.DT_BF16}[dtype_name]
+    x32 = (rng.standard_normal((T, H)) * spread).astype(np.float32)
+    if T > 1:
+        x32[T // 2] = 0
+    xt = torch.from_numpy(x32).to(tdt)
+    bits = xt.numpy() if dtype_name == "f32" else xt.view(torch.int16).numpy().view(np.uint16)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    return xt, bits, idx, code
+
+
+def _same(got, want):
+    if want is None:
+        return got is None
+    return np.array_equal(got.cpu().numpy(), want)
+
+
+QUANT_V2_CASES = [
+    # T, K, E, H, dtype
+    (3, 2, 3, 4, "f32"),
+    (64, 8, 128, 4096, "bf16"),
+    (200, 4, 16, 7168, "bf16"),
+    (100, 2, 8, 1000, "f16"),
+    (50, 3, 9, 37, "f16"),            # odd width: byte path
+    (33, 5, 10, 130, "f32"),
+]
+
+
+@pytest.mark.parametrize("T,K,E,H,dtype_name", QUANT_V2_CASES)
+def test_quant_v2_static_bit_exact(aclnn, oracle, dev, T, K, E, H, dtype_name):
+    """Static quantisation is three half-precision operations and a round-to-nearest-even: bit-exact, saturation
+    included (the spread puts a share of the values beyond +-127)."""
+    rng = np.random.default_rng(T * 7 + H)
+    xt, bits, idx, code = _quant_v2_inputs(rng, T, K, E, H, dtype_name, oracle, spread=60.0)
+    scale, offset = np.float32(0.8731), np.float32(-3.37)
+    st = torch.tensor([scale], dtype=torch.float32, device=dev)
+    ot = torch.tensor([offset], dtype=torch.float32, device=dev)
+    C = max(1, min(T, (T * K) // E))
+    for kw in (dict(expert_tokens_count_or_cumsum_flag=1), dict(expert_tokens_count_or_cumsum_flag=2, active_num=T),
+               dict(drop_pad_mode=1, expert_capacity=C, expert_tokens_before_capacity_flag=True)):
+        got = aclnn.moe_init_routing_quant_v2(xt.to(dev), torch.from_numpy(idx).to(dev), 0, st, ot, expert_num=E, **kw)
+        torch.cuda.synchronize()
+        want = oracle.moe_init_routing_quant_v2(
+            bits, idx, 0, scale, offset, active_num=kw.get("active_num", 0), expert_capacity=kw.get("expert_capacity", 0),
+            expert_num=E, drop_pad_mode=kw.get("drop_pad_mode", 0), count_flag=kw.get("expert_tokens_count_or_cumsum_flag", 0),
+            before_capacity_flag=kw.get("expert_tokens_before_capacity_flag", False), dtype=code)
+        for g, w, name in zip(got, want, ("expandedX", "expandedRowIdx", "countOrCumsum", "beforeCapacity", "dynScale")):
+            assert _same(g, w), (kw, name)
+        q = got[0].cpu().numpy()
+        assert T * H < 1000 or ((q == 127).any() and (q == -128).any())
+
+
+@pytest.mark.parametrize("T,K,E,H,dtype_name", QUANT_V2_CASES)
+@pytest.mark.parametrize("smooth_rows", [None, 1, "E"])
+def test_quant_v2_dynamic_bit_exact(aclnn, oracle, dev, T, K, E, H, dtype_name, smooth_rows):
+    """Dynamic quantisation with no smooth scale, one shared row, or one row per expert, in the dropless form, with
+    activeNum, and in the drop/pad form (unused slots keep zero rows and zero scales)."""
+    rng = np.random.default_rng(T * 11 + H)
+    xt, bits, idx, code = _quant_v2_inputs(rng, T, K, E, H, dtype_name, oracle)
+    smooth = None
+    if smooth_rows is not None:
+        smooth = (rng.random((1 if smooth_rows == 1 else E, H)) + 0.5).astype(np.float32)
+    sm_t = None if smooth is None else torch.from_numpy(smooth).to(dev)
+    C = max(1, min(T, (T * K) // E))
+    for kw in (dict(expert_tokens_count_or_cumsum_flag=2), dict(expert_tokens_count_or_cumsum_flag=1, active_num=T),
+               dict(drop_pad_mode=1, expert_capacity=C, expert_tokens_before_capacity_flag=True)):
+        got = aclnn.moe_init_routing_quant_v2(xt.to(dev), torch.from_numpy(idx).to(dev), 1, sm_t, None, expert_num=E, **kw)
+        torch.cuda.synchronize()
+        want = oracle.moe_init_routing_quant_v2(
+            bits, idx, 1, smooth, None, active_num=kw.get("active_num", 0), expert_capacity=kw.get("expert_capacity", 0),
+            expert_num=E, drop_pad_mode=kw.get("drop_pad_mode", 0), count_flag=kw.get("expert_tokens_count_or_cumsum_flag", 0),
+            before_capacity_flag=kw.get("expert_tokens_before_capacity_flag", False), dtype=code)
+        for g, w, name in zip(got, want, ("expandedX", "expandedRowIdx", "countOrCumsum", "beforeCapacity", "dynScale")):
+            assert _same(g, w), (kw, name)
+
+
+def test_quant_v2_outputs_are_rewritten_and_empty_input(aclnn, oracle, dev):
+    """Outputs that hold stale data get the same result (drop/pad zeroes its unused slots itself), and zero tokens run."""
+    rng = np.random.default_rng(5)
+    T, K, E, H, C = 40, 2, 6, 48, 20                      # capacity above what any expert receives: unused slots exist
+    xt, bits, idx, code = _quant_v2_inputs(rng, T, K, E, H, "bf16", oracle)
+    want = oracle.moe_init_routing_quant_v2(bits, idx, 1, None, None, expert_capacity=C, expert_num=E, drop_pad_mode=1,
+                                            before_capacity_flag=True, dtype=code)
+    # the binding allocates zeroed outputs; poison them through a second call on pre-filled tensors
+    h = aclnn._Handles()
+    ex = torch.full((E, C, H), 77, dtype=torch.int8, device=dev)
+    ri = torch.full((T * K,), -9, dtype=torch.int32, device=dev)
+    bef = torch.full((E,), -9, dtype=torch.int32, device=dev)
+    dyn = torch.full((E * C,), 5.0, dtype=torch.float32, device=dev)
+    x_dev, idx_dev = xt.to(dev), torch.from_numpy(idx).to(dev)         # held until the call has run
+    try:
+        args = [h.tensor(x_dev), h.tensor(idx_dev), None, None, 0, C, E, 1, 0, True, 1,
+                h.tensor(ex), h.tensor(ri), None, h.tensor(bef), h.tensor(dyn)]
+        aclnn._run_two_phase("aclnnMoeInitRoutingQuantV2", args, dev, None)
+    finally:
+        h.close()
+    torch.cuda.synchronize()
+    for g, w in zip((ex, ri, bef, dyn), (want[0], want[1], want[3], want[4])):
+        assert np.array_equal(g.cpu().numpy(), w)
+    assert (want[0].reshape(E * C, H) == 0).all(axis=1).any()          # the case does hold unused slots
+
+    empty = aclnn.moe_init_routing_quant_v2(torch.zeros((0, H), dtype=torch.bfloat16, device=dev),
+                                            torch.zeros((0, K), dtype=torch.int32, device=dev), 1, None, None,
+                                            expert_num=E, expert_tokens_count_or_cumsum_flag=1)
+    torch.cuda.synchronize()
+    assert empty[0].shape == (0, H) and empty[2].cpu().tolist() == [0] * E

@@ -229,3 +229,65 @@ def test_v3_dynamic_quant_matches_numpy(oracle, with_smooth, rng_):
     ex0, ri0, cnt0, es0 = oracle.moe_init_routing_v3_quant(x, idx, smooth, E, rng_, 2, 0)
     _, ri0_r, cnt0_r, _ = oracle.moe_init_routing_v3(x, idx, None, E, rng_, 2, 0)
     assert np.array_equal(ri0, ri0_r) and np.array_equal(cnt0, cnt0_r) and np.array_equal(ex0, ex) and np.array_equal(es0, es)
+
+
+# ------------------------------------------------------------------------------------------------ MoeInitRoutingQuantV2
+@pytest.mark.parametrize("dtype_name", ["f32", "f16", "bf16"])
+def test_quant_v2_static_matches_numpy_half_arithmetic(oracle, dtype_name):
+    """Static quantisation restated with numpy float16 arithmetic (moe_v2_gather_quant.h:93-133): numpy computes a half
+    product or sum in fp32 and rounds it to half, which equals the directly rounded result (24 >= 2 * 11 + 2 bits)."""
+    import torch
+    rng = np.random.default_rng(8)
+    T, K, E, H = 40, 3, 6, 24
+    x32 = (rng.standard_normal((T, H)) * 40).astype(np.float32)
+    x32[0, 0], x32[1, 1], x32[2, 2] = 1000.0, -2000.0, 366.0          # saturating values and one that lands near +127
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    if dtype_name == "f32":
+        bits, code, seen = x32, oracle.DT_F32, x32
+    else:
+        tdt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+        xt = torch.from_numpy(x32).to(tdt)
+        bits, seen = xt.view(torch.int16).numpy().view(np.uint16), xt.float().numpy()
+        code = oracle.DT_F16 if dtype_name == "f16" else oracle.DT_BF16
+    scale, offset = np.float32(0.3452), np.float32(1.8369)
+    ex, ri, cnt, _, dyn = oracle.moe_init_routing_quant_v2(bits, idx, 0, scale, offset, expert_num=E, count_flag=1, dtype=code)
+    _, ri_r, cnt_r, _ = oracle.moe_init_routing_v2(x32, idx, expert_num=E, count_flag=1)
+    assert dyn is None and np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r)
+    h = seen.astype(np.float16)
+    h = (h * np.float16(scale)).astype(np.float16)
+    h = (h + np.float16(offset)).astype(np.float16)
+    q = np.clip(np.rint(h.astype(np.float32)), -128, 127).astype(np.int8)
+    want = np.zeros_like(ex)
+    want[ri] = q[np.arange(T * K) // K]
+    assert np.array_equal(ex, want)
+    assert (np.abs(q.astype(np.int32)) == 127).any() or (q == -128).any()      # the saturation branch is exercised
+
+
+@pytest.mark.parametrize("smooth_rows", [0, 1, 6])
+def test_quant_v2_dynamic_equals_v3_dynamic_and_drop_pad(oracle, smooth_rows):
+    rng = np.random.default_rng(12)
+    T, K, E, H = 50, 2, 6, 20
+    x = (rng.standard_normal((T, H)) * 3).astype(np.float32)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    smooth = None if smooth_rows == 0 else (rng.random((smooth_rows, H)) + 0.5).astype(np.float32)
+    ex, ri, _, _, dyn = oracle.moe_init_routing_quant_v2(x, idx, 1, smooth, expert_num=E)
+    full = None if smooth is None else np.broadcast_to(smooth, (E, H)).copy()
+    ex3, ri3, _, es3 = oracle.moe_init_routing_v3_quant(x, idx, full, E, None, 1, 1)
+    assert np.array_equal(ex, ex3) and np.array_equal(ri, ri3) and np.array_equal(dyn, es3)
+    # drop/pad: rows land at expert * capacity + rank, the rest is zero with scale 0
+    C = 5
+    exd, rid, _, bef, dynd = oracle.moe_init_routing_quant_v2(x, idx, 1, smooth, expert_capacity=C, expert_num=E,
+                                                              drop_pad_mode=1, before_capacity_flag=True)
+    _, rid_r, _, bef_r = oracle.moe_init_routing_v2(x, idx, expert_capacity=C, expert_num=E, drop_pad_mode=1,
+                                                    before_capacity_flag=True)
+    assert np.array_equal(rid, rid_r) and np.array_equal(bef, bef_r)
+    flat = exd.reshape(E * C, H)
+    used = np.zeros(E * C, bool)
+    for i in range(T * K):
+        if rid[i] >= 0:
+            used[rid[i]] = True
+            assert np.array_equal(flat[rid[i]], ex[ri[i]]) and dynd[rid[i]] == dyn[ri[i]]
+    assert not flat[~used].any() and not dynd[~used].any()
+    # activeNum cuts the dropless output
+    exa, _, _, _, dyna = oracle.moe_init_routing_quant_v2(x, idx, 1, smooth, active_num=37, expert_num=E)
+    assert exa.shape == (37, H) and np.array_equal(exa, ex[:37]) and np.array_equal(dyna, dyn[:37])
