@@ -5,6 +5,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <new>
 
 #include "opapi_profile.h"
@@ -27,7 +28,11 @@ void SetError(const char* fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(buf, sizeof(buf), fmt, ap);
     va_end(ap);
-    g_lastError = buf;
+    try {
+        g_lastError = buf;
+    } catch (...) {  // out of host memory: the status code still reaches the caller, the text does not
+        g_lastError.clear();
+    }
     if (const char* v = std::getenv("OPAPI_LOG_ERRORS")) {
         if (v[0] != '\0' && v[0] != '0') fprintf(stderr, "[opapi] %s\n", buf);
     }
@@ -79,9 +84,10 @@ struct TimedLaunch {
     hipEvent_t start, stop;
 };
 bool g_timerOn = false;
+std::mutex g_timedMutex;  // guards g_timed: operators may be enqueued from several host threads
 std::vector<TimedLaunch> g_timed;
 
-void DropTimed() {
+void DropTimed() {  // caller holds g_timedMutex
     for (TimedLaunch& t : g_timed) {
         (void)hipEventDestroy(t.start);
         (void)hipEventDestroy(t.stop);
@@ -101,7 +107,13 @@ KernelTimer::~KernelTimer() {
     hipEvent_t stop = nullptr;
     if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start_); return; }
     (void)hipEventRecord(stop, stream_);
-    g_timed.push_back({name_, start_, stop});
+    try {
+        std::lock_guard<std::mutex> lock(g_timedMutex);
+        g_timed.push_back({name_, start_, stop});
+    } catch (...) {  // out of host memory: this launch goes untimed
+        (void)hipEventDestroy(start_);
+        (void)hipEventDestroy(stop);
+    }
 }
 
 }  // namespace opapi
@@ -109,11 +121,13 @@ KernelTimer::~KernelTimer() {
 extern "C" {
 
 void opapiKernelTimerEnable(int enable) {
+    std::lock_guard<std::mutex> lock(opapi::g_timedMutex);
     opapi::DropTimed();
     opapi::g_timerOn = enable != 0;
 }
 
-int opapiKernelTimerReport(char* buf, size_t cap) {
+int opapiKernelTimerReport(char* buf, size_t cap) try {
+    std::lock_guard<std::mutex> lock(opapi::g_timedMutex);
     std::map<std::string, std::pair<int, double>> agg;
     int rc = 0;
     for (opapi::TimedLaunch& t : opapi::g_timed) {
@@ -136,6 +150,8 @@ int opapiKernelTimerReport(char* buf, size_t cap) {
         buf[n] = '\0';
     }
     return rc < 0 ? rc : static_cast<int>(agg.size());
+} catch (...) {  // out of host memory while building the report
+    return -1;
 }
 
 aclError aclInit(const char*) { return ACL_SUCCESS; }
@@ -182,16 +198,24 @@ aclTensor* aclCreateTensor(const int64_t* viewDims, uint64_t viewDimsNum, aclDat
                            int64_t offset, aclFormat format, const int64_t* storageDims, uint64_t storageDimsNum,
                            void* tensorData) {
     if ((viewDimsNum > 0 && viewDims == nullptr) || viewDimsNum > 8 || storageDimsNum > 8) return nullptr;
+    for (uint64_t i = 0; i < viewDimsNum; ++i) {
+        if (viewDims[i] < 0) return nullptr;
+    }
     aclTensor* t = new (std::nothrow) aclTensor();
     if (t == nullptr) return nullptr;
-    t->dims.assign(viewDims, viewDims + viewDimsNum);
-    if (stride != nullptr) {
-        t->strides.assign(stride, stride + viewDimsNum);
-    } else {  // contiguous default
-        t->strides.assign(viewDimsNum, 1);
-        for (int i = (int)viewDimsNum - 2; i >= 0; --i) t->strides[i] = t->strides[i + 1] * t->dims[i + 1];
+    try {  // no exception may cross the C boundary
+        t->dims.assign(viewDims, viewDims + viewDimsNum);
+        if (stride != nullptr) {
+            t->strides.assign(stride, stride + viewDimsNum);
+        } else {  // contiguous default
+            t->strides.assign(viewDimsNum, 1);
+            for (int i = (int)viewDimsNum - 2; i >= 0; --i) t->strides[i] = t->strides[i + 1] * t->dims[i + 1];
+        }
+        if (storageDims != nullptr) t->storage.assign(storageDims, storageDims + storageDimsNum);
+    } catch (...) {
+        delete t;
+        return nullptr;
     }
-    if (storageDims != nullptr) t->storage.assign(storageDims, storageDims + storageDimsNum);
     t->offset = offset;
     t->dtype = dataType;
     t->format = format;
@@ -206,7 +230,12 @@ aclTensorList* aclCreateTensorList(const aclTensor* const* value, uint64_t size)
     if (size > 0 && value == nullptr) return nullptr;
     aclTensorList* l = new (std::nothrow) aclTensorList();
     if (l == nullptr) return nullptr;
-    l->items.assign(value, value + size);
+    try {
+        l->items.assign(value, value + size);
+    } catch (...) {
+        delete l;
+        return nullptr;
+    }
     return l;
 }
 aclnnStatus aclDestroyTensorList(const aclTensorList* tensorList) {
@@ -220,7 +249,12 @@ aclIntArray* aclCreateIntArray(const int64_t* value, uint64_t size) {
     if (size > 0 && value == nullptr) return nullptr;
     aclIntArray* a = new (std::nothrow) aclIntArray();
     if (a == nullptr) return nullptr;
-    a->values.assign(value, value + size);
+    try {
+        a->values.assign(value, value + size);
+    } catch (...) {
+        delete a;
+        return nullptr;
+    }
     return a;
 }
 aclnnStatus aclDestroyIntArray(const aclIntArray* array) {
