@@ -198,9 +198,6 @@ aclTensor* aclCreateTensor(const int64_t* viewDims, uint64_t viewDimsNum, aclDat
                            int64_t offset, aclFormat format, const int64_t* storageDims, uint64_t storageDimsNum,
                            void* tensorData) {
     if ((viewDimsNum > 0 && viewDims == nullptr) || viewDimsNum > 8 || storageDimsNum > 8) return nullptr;
-    for (uint64_t i = 0; i < viewDimsNum; ++i) {
-        if (viewDims[i] < 0) return nullptr;
-    }
     aclTensor* t = new (std::nothrow) aclTensor();
     if (t == nullptr) return nullptr;
     try {  // no exception may cross the C boundary
