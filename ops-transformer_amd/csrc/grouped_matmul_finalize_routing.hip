@@ -114,6 +114,7 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
                 "%s do not support input nullptr (x1, x2, scale, groupList, rowIndex, out).", api);
     OPAPI_CHECK_NOTNULL(workspaceSize, "workspaceSize");
     OPAPI_CHECK_NOTNULL(executor, "executor");
+    OPAPI_CHECK_EXTENTS(x1, x2, scale, bias, perToken, groupList, sharedInput, logit, rowIndex, out);
     OPAPI_CHECK(antiquantScale == nullptr && antiquantOffset == nullptr, ACLNN_ERR_PARAM_NULLPTR,
                 "%s: antiquantScale / antiquantOffset are not enabled and must be nullptr.", api);
     OPAPI_CHECK(dtype == 0, kInvalid, "%s dtype must be 0, but is %lld.", api, (long long)dtype);

@@ -59,6 +59,7 @@ aclnnStatus PlanSwigluQuant(const aclTensor* x, const aclTensor* weight, const a
     OPAPI_CHECK_NOTNULL(outputScale, "outputScale");
     OPAPI_CHECK_NOTNULL(workspaceSize, "workspaceSize");
     OPAPI_CHECK_NOTNULL(executor, "executor");
+    OPAPI_CHECK_EXTENTS(x, weight, weightScale, xScale, groupList, output, outputScale);
     constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;
 
     OPAPI_CHECK(x->dtype == ACL_INT8 && weight->dtype == ACL_INT8, kInvalid,

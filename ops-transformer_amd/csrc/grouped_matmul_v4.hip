@@ -121,6 +121,7 @@ aclnnStatus PlanGroupedMatmul(
     OPAPI_CHECK(xt != nullptr, kInvalid, "x[0] is nullptr!");
     OPAPI_CHECK(wt != nullptr, kInvalid, "weight[0] is nullptr!");
     OPAPI_CHECK(yt != nullptr, kInvalid, "y[0] is nullptr!");
+    OPAPI_CHECK_EXTENTS(xt, wt, yt, groupListOptional);
     OPAPI_CHECK(xt->dtype == ACL_INT8 && wt->dtype == ACL_INT8, kInvalid,
                 "only INT8 x and INT8 weight are built (got %d, %d)", (int)xt->dtype, (int)wt->dtype);
     // A blocked (FRACTAL_NZ) int8 weight is [E, N/32, K/16, 16, 32], given as that 5-D tensor or as the 3-D view

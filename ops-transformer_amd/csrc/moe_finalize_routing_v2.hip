@@ -193,6 +193,7 @@ extern "C" aclnnStatus aclnnMoeFinalizeRoutingV2GetWorkspaceSize(
     OPAPI_CHECK_NOTNULL(out, "out");
     OPAPI_CHECK_NOTNULL(workspaceSize, "workspaceSize");
     OPAPI_CHECK_NOTNULL(executor, "executor");
+    OPAPI_CHECK_EXTENTS(expandedX, expandedRowIdx, x1Optional, x2Optional, biasOptional, scalesOptional, expertIdxOptional, out);
     constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;
 
     const aclDataType dt = expandedX->dtype;

@@ -259,6 +259,7 @@ extern "C" aclnnStatus aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize(
     OPAPI_CHECK_NOTNULL(expertIdxOut, "expertIdxOut");
     OPAPI_CHECK_NOTNULL(workspaceSize, "workspaceSize");
     OPAPI_CHECK_NOTNULL(executor, "executor");
+    OPAPI_CHECK_EXTENTS(x, finishedOptional, yOut, expertIdxOut, softmaxResultOutOptional);
 
     constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;
     OPAPI_CHECK(x->dtype == ACL_FLOAT || x->dtype == ACL_FLOAT16 || x->dtype == ACL_BF16, kInvalid,

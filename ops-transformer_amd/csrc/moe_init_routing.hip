@@ -790,6 +790,9 @@ aclnnStatus PlanRoutingV2(const aclTensor* x, const aclTensor* expertIdx, const 
     int64_t countFlag = dropPadMode == 1 ? 0 : expertTokensCountOrCumsumFlag;
     bool beforeFlag = dropPadMode == 1 ? expertTokensBeforeCapacityFlag : false;
 
+    // after the attribute rules, so that a negative activeNum is reported as such and not through the shapes built on it
+    OPAPI_CHECK_EXTENTS(x, expertIdx, scaleOptional, offsetOptional, expandedXOut, expandedRowIdxOut, expertTokensCountOrCumsumOut,
+                        expertTokensBeforeCapacityOut, dynamicQuantScaleOut);
     const int64_t tokens = x->dims[0], cols = x->dims[1], topK = expertIdx->dims[1];
     const int64_t total = tokens * topK;
     OPAPI_CHECK(total < (1ll << 31), kInvalid, "tokens * topK = %lld does not fit int32 row indices", (long long)total);
@@ -960,6 +963,7 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
     OPAPI_CHECK_NOTNULL(expertTokensCountOrCumsumOut, "expertTokensCountOrCumsumOut");
     OPAPI_CHECK_NOTNULL(workspaceSize, "workspaceSize");
     OPAPI_CHECK_NOTNULL(executor, "executor");
+    OPAPI_CHECK_EXTENTS(x, expertIdx, scaleOptional, expandedXOut, expandedRowIdxOut, expertTokensCountOrCumsumOut, expandedScaleOut);
     (void)expertCapacity;  // unused by the reference as well (dropless only)
 
     constexpr aclnnStatus kInvalid = ACLNN_ERR_PARAM_INVALID;

@@ -64,6 +64,15 @@ inline int64_t Numel(const aclTensor* t) {
 
 inline bool IsEmpty(const aclTensor* t) { return t == nullptr || Numel(t) == 0; }
 
+// Extents are caller data: a negative one would make every size derived from it meaningless.
+inline bool HasNegativeDim(const aclTensor* t) {
+    if (t == nullptr) return false;
+    for (int64_t d : t->dims) {
+        if (d < 0) return true;
+    }
+    return false;
+}
+
 // Row-major contiguous view (dims of extent 1 may carry any stride).
 inline bool IsContiguous(const aclTensor* t) {
     int64_t expect = 1;
@@ -121,6 +130,16 @@ class KernelTimer {
             ::opapi::SetError(__VA_ARGS__);     \
             return (code);                      \
         }                                       \
+    } while (0)
+
+// Rejects tensors (absent ones pass) that carry a negative extent.
+#define OPAPI_CHECK_EXTENTS(...)                                                                              \
+    do {                                                                                                      \
+        const aclTensor* const opapiTensors_[] = {__VA_ARGS__};                                               \
+        for (const aclTensor* opapiT_ : opapiTensors_) {                                                      \
+            OPAPI_CHECK(!::opapi::HasNegativeDim(opapiT_), ACLNN_ERR_PARAM_INVALID,                           \
+                        "%s: a tensor has a negative extent: %s", __func__, ::opapi::ShapeStr(opapiT_).c_str()); \
+        }                                                                                                     \
     } while (0)
 
 #define OPAPI_CHECK_NOTNULL(ptr, name) \

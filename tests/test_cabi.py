@@ -640,3 +640,21 @@ def test_second_phase_rejects_bad_workspace(aclnn):
     st = lib.aclnnMoeInitRoutingV2(None, ws.value, ex, None)   # null workspace although bytes are required
     assert st == NULLPTR
     assert lib.aclnnMoeInitRoutingV2(None, 0, None, None) == NULLPTR  # null executor
+
+
+# ------------------------------------------------------------------------------------------------ negative extents
+def test_negative_extents_are_rejected_everywhere(aclnn):
+    """Shapes are caller data: a set of tensors that agree with each other on a negative extent is still refused."""
+    cases = [
+        ("aclnnMoeInitRoutingV2", _routing_args(aclnn, T_=-4)),
+        ("aclnnMoeInitRoutingQuantV2", _routing_quant_v2_args(aclnn, T_=-4)),
+        ("aclnnMoeInitRoutingV3", _routing_v3_args(aclnn, T_=-4, active=-1)),
+        ("aclnnMoeGatingTopKSoftmaxV2", _gating_args(aclnn, shape=(-6, 16))),
+        ("aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=-192)),
+        ("aclnnGroupedMatmulV4", _gmm_args(aclnn, M=-64)),
+        _combine_args(aclnn, M=-64),
+        ("aclnnMoeFinalizeRoutingV2", _fin_args(aclnn, T_=-12)),
+    ]
+    for api, args in cases:
+        code, msg = _status(aclnn, api, args)
+        assert code == INVALID and "negative extent" in msg, (api, code, msg)
