@@ -224,6 +224,94 @@ __global__ __launch_bounds__(kSortThreads) void DigitScatterKernel(SortPass p, I
     }
 }
 
+// Small inputs (decode steps): histogram, scan and scatter of a single-pass sort in ONE workgroup, so the sort costs one
+// launch instead of three.  Sixteen waves take one slice of the keys each; the per-wave tables and the digit offsets
+// stay in LDS.  Writes everything the three kernels above write (binBase / binTotal included: later kernels read them).
+constexpr int kSmallSortWaves = 16;
+constexpr int kSmallSortBins = 512;
+constexpr int64_t kSmallSortMaxKeys = 8192;
+
+__global__ __launch_bounds__(kSmallSortWaves * kWaveSize) void SmallSortKernel(SortPass p, CountOutputs co, InverseMap im) {
+    __shared__ int32_t tbl[kSmallSortWaves][kSmallSortBins];
+    __shared__ int32_t base[kSmallSortBins];   // exclusive offset of each digit value
+    __shared__ int32_t scan[kSmallSortBins];
+    const int lane = threadIdx.x % kWaveSize;
+    const int wave = threadIdx.x / kWaveSize;
+    const int bins = 1 << p.bits;              // <= kSmallSortBins
+    const int64_t begin = static_cast<int64_t>(wave) * p.sliceLen;
+
+    for (int b = lane; b < bins; b += kWaveSize) tbl[wave][b] = 0;
+    WaveSync();
+    for (int off = 0; off < p.sliceLen; off += kWaveSize) {
+        const int64_t i = begin + off + lane;
+        const bool valid = i < p.total;
+        const uint32_t digit = valid ? DigitOf(p.keysIn[i], p) : 0u;
+        const uint64_t mask = MatchDigit(digit, p.bits, valid);
+        if (valid && lane == __ffsll(static_cast<unsigned long long>(mask)) - 1) tbl[wave][digit] += __popcll(mask);
+        WaveSync();
+    }
+    __syncthreads();
+
+    // thread b < bins: the slices' counts of digit value b become exclusive prefixes, their sum the value's total
+    const int b = threadIdx.x;
+    int32_t total = 0;
+    if (b < bins) {
+        for (int w = 0; w < kSmallSortWaves; ++w) {
+            const int32_t v = tbl[w][b];
+            tbl[w][b] = total;
+            total += v;
+        }
+        scan[b] = total;
+    }
+    __syncthreads();
+    for (int d = 1; d < bins; d <<= 1) {
+        const int32_t add = (b < bins && b >= d) ? scan[b - d] : 0;
+        __syncthreads();
+        if (b < bins) scan[b] += add;
+        __syncthreads();
+    }
+    if (b < bins) {
+        const int32_t mine = scan[b] - total;
+        base[b] = mine;
+        p.binBase[b] = mine;
+        p.binTotal[b] = total;
+        if (b < co.expertNum) {
+            if (co.countOrCumsum != nullptr) co.countOrCumsum[b] = co.flag == 1 ? mine + total : total;
+            if (co.beforeCapacity != nullptr) co.beforeCapacity[b] = total;
+            if (co.wide != nullptr) co.wide[b] = co.wideCumsum ? mine + total : total;
+        }
+    }
+    __syncthreads();
+
+    const uint64_t lanesBelow = (1ull << lane) - 1ull;
+    const int32_t dropBase = im.dropFrom >= 0 ? base[im.dropFrom] : 0;
+    for (int off = 0; off < p.sliceLen; off += kWaveSize) {
+        const int64_t i = begin + off + lane;
+        const bool valid = i < p.total;
+        const int32_t key = valid ? p.keysIn[i] : 0;
+        const uint32_t digit = valid ? DigitOf(key, p) : 0u;
+        const uint64_t mask = MatchDigit(digit, p.bits, valid);
+        int32_t dst = 0;
+        if (valid) dst = base[digit] + tbl[wave][digit] + __popcll(mask & lanesBelow);
+        WaveSync();
+        if (valid && lane == __ffsll(static_cast<unsigned long long>(mask)) - 1) tbl[wave][digit] += __popcll(mask);
+        WaveSync();
+        if (valid) {
+            const int32_t payload = static_cast<int32_t>(i);
+            const bool dropped = im.dropFrom >= 0 && dst >= dropBase;
+            if (im.expandedRowIdx != nullptr) {
+                int32_t row = dst;
+                if (im.dropPad) {
+                    const int32_t rank = dst - base[digit];
+                    row = rank < im.capacity ? static_cast<int32_t>(digit) * im.capacity + rank : -1;
+                }
+                im.expandedRowIdx[payload] = dropped ? -1 : row;
+            }
+            if (im.gatherIdx != nullptr) im.gatherIdx[dst] = dropped ? -1 : payload;
+        }
+    }
+}
+
 // Per-expert cumsum / count from fully sorted keys, for id ranges wider than one digit:
 // cumsum[e] = number of sorted keys <= e (upper bound).
 __global__ void CountFromSortedKernel(const int32_t* sortedKeys, int64_t total, CountOutputs co) {
@@ -554,6 +642,7 @@ class InitRoutingExecutor : public aclOpExecutor {
     int keyBits = 0;
     bool signedRange = false;  // id range unknown: sort all 32 bits, sign-aware
     int32_t sliceLen = 0, numSlices = 0;
+    bool smallSort = false;
     uint64_t offKeys[2] = {0, 0}, offPayload[2] = {0, 0}, offTable = 0, offBinBase = 0, offBinTotal = 0;
 
     void Plan() {
@@ -578,6 +667,15 @@ class InitRoutingExecutor : public aclOpExecutor {
         sliceLen = static_cast<int32_t>(len);
         numSlices = static_cast<int32_t>((total + len - 1) / len);
         if (numSlices < 1) numSlices = 1;
+        // decode-sized inputs: the whole single-pass sort in one workgroup, one slice per wave
+        smallSort = passes == 1 && bitsPerPass[0] <= CeilLog2(kSmallSortBins) && total <= kSmallSortMaxKeys;
+        if (smallSort) {
+            len = (total + kSmallSortWaves - 1) / kSmallSortWaves;
+            len = (len + kWaveSize - 1) / kWaveSize * kWaveSize;
+            if (len < kWaveSize) len = kWaveSize;
+            sliceLen = static_cast<int32_t>(len);
+            numSlices = kSmallSortWaves;
+        }
 
         uint64_t off = 0;
         auto take = [&](uint64_t bytes) {
@@ -670,6 +768,11 @@ class InitRoutingExecutor : public aclOpExecutor {
             }
             InverseMap im{last ? expandedRowIdx : nullptr, dropPad, static_cast<int32_t>(capacity),
                           last ? gatherIdxOut : nullptr, (remap && passes == 1) ? expertEnd - expertStart : -1};
+            if (smallSort) {
+                opapi::KernelTimer timer("routing_small_sort", stream);
+                hipLaunchKernelGGL(SmallSortKernel, dim3(1), dim3(kSmallSortWaves * kWaveSize), 0, stream, p, co, im);
+                break;
+            }
             {
                 opapi::KernelTimer timer("routing_histogram", stream);
                 hipLaunchKernelGGL(DigitHistogramKernel, dim3(sortBlocks), dim3(kSortThreads), 0, stream, p);

@@ -22,6 +22,9 @@ CASES = [  # T, K, E, H, dtype
     (1000, 4, 33, 18, np.int8),        # 18-byte rows: 2-byte vector path
     (4096, 8, 256, 512, np.float16),   # DeepSeek-V3 routing shape (narrow rows keep the host copy small)
     (2048, 6, 2000, 8, np.float32),    # 11-bit digit
+    (1024, 8, 512, 16, np.int8),       # 8192 keys, 512 experts: the largest input the one-workgroup sort takes
+    (8193, 1, 512, 4, np.int8),        # one key more: the three-kernel sort
+    (1000, 8, 513, 4, np.int8),        # one expert more: ten digit bits, the three-kernel sort
 ]
 
 
