@@ -126,3 +126,43 @@ def test_nz_weight_chain_equals_nd_chain(pkg, dev):
     b = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, weight_nz=True).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
     torch.cuda.synchronize()
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_two_host_threads_on_their_own_streams(pkg, dev):
+    """All state of a call lives in its executor: two host threads that run the chain at the same time, each on its own
+    stream with its own buffers, both get the single-threaded result bit for bit (ctypes drops the interpreter lock
+    during the calls, so the first and second phases of the two threads do interleave)."""
+    import threading
+    cfg = pkg.synth.config(0)
+    w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=0)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    inputs, expected = [], []
+    for seed in (11, 12):
+        idx, wgt = pkg.synth.make_routing(cfg, seed=seed)
+        xq, xs = pkg.synth.make_activations(cfg, seed=seed)
+        args = (t(xq), t(xs), t(idx), t(wgt))
+        inputs.append(args)
+        expected.append(pkg.MoeFfnW8A8(w13, w13s, w2, w2s).forward(*args).clone())
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream(device=dev)
+            ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s)
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    out = ffn.forward(*inputs[i])
+                results[i] = out.clone()
+            stream.synchronize()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not errors, errors
+    for got, want in zip(results, expected):
+        assert got is not None and torch.equal(got, want)
