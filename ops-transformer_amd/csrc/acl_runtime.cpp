@@ -50,6 +50,67 @@ std::string ShapeStr(const aclTensor* t) {
     return s + "]";
 }
 
+}  // namespace opapi
+
+aclnnStatus aclOpExecutor::BindRaw(const aclTensor* t, void* slotAddr, const void** now) {
+    *now = nullptr;
+    if (t == nullptr) return ACLNN_SUCCESS;
+    *now = opapi::DataPtr(t);
+    if (opapi::Numel(t) == 0 || opapi::IsContiguous(t)) return ACLNN_SUCCESS;
+    opapi::StagedInput s;
+    s.slotAddr = slotAddr;
+    s.offset = stagingBytes;
+    s.src = opapi::DataPtr(t);
+    s.numel = opapi::Numel(t);
+    s.nd = static_cast<int32_t>(t->dims.size());
+    s.elemSize = static_cast<int32_t>(opapi::ElemSize(t->dtype));
+    OPAPI_CHECK(s.nd <= 8 && t->strides.size() == t->dims.size(), ACLNN_ERR_PARAM_INVALID,
+                "a non-contiguous input has more than 8 dimensions or no strides");
+    OPAPI_CHECK(s.elemSize > 0, ACLNN_ERR_PARAM_INVALID, "a non-contiguous input has an unsupported data type");
+    for (int d = 0; d < s.nd; ++d) {
+        OPAPI_CHECK(t->strides[d] >= 0, ACLNN_ERR_PARAM_INVALID, "negative strides are not supported (%s)",
+                    opapi::ShapeStr(t).c_str());
+        s.dims[d] = t->dims[d];
+        s.strides[d] = t->strides[d];
+    }
+    OPAPI_CHECK(t->data != nullptr, ACLNN_ERR_PARAM_NULLPTR, "a tensor carries no device memory");
+    try {
+        staged.push_back(s);
+    } catch (...) {
+        opapi::SetError("out of host memory");
+        return ACLNN_ERR_INNER;
+    }
+    stagingBytes += (static_cast<uint64_t>(s.numel) * static_cast<uint64_t>(s.elemSize) + 255) / 256 * 256;
+    // aligned stand-in until the second phase knows the workspace address
+    *now = reinterpret_cast<const void*>(static_cast<uintptr_t>(1) << 20);
+    return ACLNN_SUCCESS;
+}
+
+namespace opapi {
+
+namespace {
+// dst[i] = src[sum_d index_d(i) * stride_d], i running over the view in row-major order; one element per thread.
+template <typename T>
+__global__ void StridedCopyKernel(StagedInput s, T* dst) {
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < s.numel; i += step) {
+        int64_t rest = i, off = 0;
+        for (int d = s.nd - 1; d >= 0; --d) {
+            off += (rest % s.dims[d]) * s.strides[d];
+            rest /= s.dims[d];
+        }
+        dst[i] = reinterpret_cast<const T*>(s.src)[off];
+    }
+}
+
+template <typename T>
+void LaunchStridedCopy(const StagedInput& s, void* dst, hipStream_t stream) {
+    int64_t blocks = (s.numel + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(StridedCopyKernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, s, static_cast<T*>(dst));
+}
+}  // namespace
+
 aclnnStatus RunAndRelease(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor, aclrtStream stream) {
     if (executor == nullptr) {
         SetError("second-phase call: executor must not be null");
@@ -64,7 +125,22 @@ aclnnStatus RunAndRelease(void* workspace, uint64_t workspaceSize, aclOpExecutor
         SetError("second-phase call: workspaceSize %llu is smaller than the required %llu",
                  (unsigned long long)workspaceSize, (unsigned long long)executor->workspaceBytes);
         st = ACLNN_ERR_PARAM_INVALID;
+    } else if (!executor->staged.empty() && reinterpret_cast<uintptr_t>(workspace) % 256 != 0) {
+        SetError("second-phase call: the workspace must be 256-byte aligned when non-contiguous inputs are staged in it");
+        st = ACLNN_ERR_PARAM_INVALID;
     } else {
+        for (const StagedInput& s : executor->staged) {
+            char* const dst = static_cast<char*>(workspace) + executor->stagingBase + s.offset;
+            KernelTimer timer("stage_input", static_cast<hipStream_t>(stream));
+            switch (s.elemSize) {
+                case 1: LaunchStridedCopy<uint8_t>(s, dst, static_cast<hipStream_t>(stream)); break;
+                case 2: LaunchStridedCopy<uint16_t>(s, dst, static_cast<hipStream_t>(stream)); break;
+                case 4: LaunchStridedCopy<uint32_t>(s, dst, static_cast<hipStream_t>(stream)); break;
+                default: LaunchStridedCopy<uint64_t>(s, dst, static_cast<hipStream_t>(stream)); break;
+            }
+            void* const patched = dst;
+            memcpy(s.slotAddr, &patched, sizeof(void*));
+        }
         st = executor->Run(workspace, static_cast<hipStream_t>(stream));
         if (st == ACLNN_SUCCESS) {
             hipError_t e = hipGetLastError();

@@ -84,6 +84,8 @@ class CombineExecutor : public aclOpExecutor {
             else hipLaunchKernelGGL(InitCombineOutputKernel<1>, dim3(blocks), dim3(256), 0, stream, init);
         }
         if (problem.M == 0) return ACLNN_SUCCESS;
+        problem.combineWeight = logit;
+        problem.rowScale = perToken;
         if (needRowFactor) {
             float* rowFactor = reinterpret_cast<float*>(ws + offRowFactor);
             hipLaunchKernelGGL(RowFactorKernel, dim3(static_cast<unsigned>((problem.M + 255) / 256)), dim3(256), 0, stream,
@@ -208,10 +210,7 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
     const bool wTransposed = !nz && IsLastTwoDimsTransposed(x2);
     OPAPI_CHECK(nz || wTransposed || IsContiguous(x2), kInvalid,
                 "x2 must be contiguous [E,K,N] or the transposed view of contiguous [E,N,K] storage");
-    const aclTensor* plain[] = {x1, scale, bias, perToken, groupList, sharedInput, logit, rowIndex, out};
-    for (const aclTensor* t : plain) {
-        OPAPI_CHECK(t == nullptr || IsContiguous(t), kInvalid, "all tensors other than x2 must be contiguous");
-    }
+    OPAPI_CHECK(IsContiguous(out), kInvalid, "out must be contiguous");  // inputs other than x2 may be strided views
     const aclTensor* all[] = {x1, x2, scale, bias, perToken, groupList, sharedInput, logit, rowIndex, out};
     for (const aclTensor* t : all) {
         OPAPI_CHECK(t == nullptr || Numel(t) == 0 || t->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
@@ -221,17 +220,17 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
     auto* ex = new (std::nothrow) CombineExecutor();
     OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
     ex->init.out = reinterpret_cast<float*>(DataPtr(out));
-    ex->init.shared = reinterpret_cast<const uint16_t*>(DataPtr(sharedInput));
+    OPAPI_BIND(ex, sharedInput, &ex->init.shared);
     ex->init.sharedIsBf16 = sharedInput != nullptr && sharedInput->dtype == ACL_BF16 ? 1 : 0;
     ex->init.sharedWeight = sharedInputWeight;
     ex->init.sharedOffset = sharedInputOffset;
     ex->init.sharedRows = sharedRows;
     ex->init.batch = batch;
     ex->init.n = n;
-    ex->perToken = reinterpret_cast<const float*>(DataPtr(perToken));
-    ex->logit = reinterpret_cast<const float*>(DataPtr(logit));
+    OPAPI_BIND(ex, perToken, &ex->perToken);
+    OPAPI_BIND(ex, logit, &ex->logit);
     gemm::Problem& p = ex->problem;
-    p.x = reinterpret_cast<const int8_t*>(DataPtr(x1));
+    OPAPI_BIND(ex, x1, &p.x);
     p.w = reinterpret_cast<const int8_t*>(DataPtr(x2));
     p.wKMajor = wTransposed;
     p.wNz = nz;
@@ -239,20 +238,20 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
     p.K = k;
     p.N = n;
     p.groups = static_cast<int32_t>(e);
-    p.groupList = DataPtr(groupList);
+    OPAPI_BIND(ex, groupList, &p.groupList);
     p.groupListIsInt64 = groupList->dtype == ACL_INT64;
     p.groupListKind = groupListType == 1 ? gemm::GroupListKind::kCount : gemm::GroupListKind::kCumsum;
     p.expectedRowsPerGroup = expected;
     p.epilogue = gemm::Epilogue::kDequant;
     p.out = DataPtr(out);
     p.outDtype = static_cast<int>(ACL_FLOAT);
-    p.scale = DataPtr(scale);
+    OPAPI_BIND(ex, scale, &p.scale);
     p.scaleDtype = static_cast<int>(scale->dtype);
-    p.combineIndex = DataPtr(rowIndex);
+    OPAPI_BIND(ex, rowIndex, &p.combineIndex);
     p.combineIndexIsInt64 = rowIndex->dtype == ACL_INT64;
     p.combineRows = batch;
-    p.combineWeight = ex->logit;
-    p.bias = DataPtr(bias);
+    p.combineWeight = ex->logit;  // both refreshed in Run, where staged inputs have their final address
+    OPAPI_BIND(ex, bias, &p.bias);
     p.biasDtype = bias != nullptr ? static_cast<int>(bias->dtype) : 0;
     ex->plan = gemm::MakePlan(p);
     // the row factor: perToken alone can be used as it is; anything involving logit is multiplied out first
@@ -263,7 +262,7 @@ aclnnStatus PlanCombine(const char* api, const aclTensor* x1, const aclTensor* x
         ex->offRowFactor = AlignUp(bytes, 256);
         bytes = ex->offRowFactor + AlignUp(static_cast<uint64_t>(m) * 4, 256);
     }
-    ex->workspaceBytes = p.M == 0 ? 0 : bytes;
+    ex->SealWorkspace(p.M == 0 ? 0 : bytes);
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;

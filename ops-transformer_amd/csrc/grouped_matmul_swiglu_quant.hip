@@ -134,9 +134,8 @@ aclnnStatus PlanSwigluQuant(const aclTensor* x, const aclTensor* weight, const a
     OPAPI_CHECK(nz || wTransposed || IsContiguous(weight), kInvalid,
                 "weight must be contiguous [E,K,N] or the transposed view of contiguous [E,N,K] storage");
     OPAPI_CHECK(!nz || weight->offset == 0, kInvalid, "a FRACTAL_NZ weight must start at its storage");
-    OPAPI_CHECK(IsContiguous(x) && IsContiguous(weightScale) && IsContiguous(xScale) && IsContiguous(groupList) &&
-                    IsContiguous(output) && IsContiguous(outputScale),
-                kInvalid, "x, weightScale, xScale, groupList, output and outputScale must be contiguous");
+    OPAPI_CHECK(IsContiguous(output) && IsContiguous(outputScale), kInvalid,
+                "output and outputScale must be contiguous");  // the inputs other than weight may be strided views
     const aclTensor* all[] = {x, weight, weightScale, xScale, groupList, output, outputScale};
     for (const aclTensor* t : all) {
         OPAPI_CHECK(t->data != nullptr, ACLNN_ERR_PARAM_NULLPTR, "a tensor carries no device memory");
@@ -145,7 +144,7 @@ aclnnStatus PlanSwigluQuant(const aclTensor* x, const aclTensor* weight, const a
     auto* ex = new (std::nothrow) SwigluQuantExecutor();
     OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
     gemm::Problem& p = ex->problem;
-    p.x = reinterpret_cast<const int8_t*>(DataPtr(x));
+    OPAPI_BIND(ex, x, &p.x);
     p.w = reinterpret_cast<const int8_t*>(DataPtr(weight));
     p.wKMajor = wTransposed;
     p.wNz = nz;
@@ -153,17 +152,17 @@ aclnnStatus PlanSwigluQuant(const aclTensor* x, const aclTensor* weight, const a
     p.K = k;
     p.N = n;
     p.groups = static_cast<int32_t>(groupListLen);
-    p.groupList = DataPtr(groupList);
+    OPAPI_BIND(ex, groupList, &p.groupList);
     p.groupListIsInt64 = groupList->dtype == ACL_INT64;
     p.groupListKind = gemm::GroupListKind::kCumsum;
     p.epilogue = gemm::Epilogue::kSwiglu;
-    p.scale = DataPtr(weightScale);
+    OPAPI_BIND(ex, weightScale, &p.scale);
     p.scaleDtype = static_cast<int>(weightScale->dtype);
-    p.rowScale = reinterpret_cast<const float*>(DataPtr(xScale));
+    OPAPI_BIND(ex, xScale, &p.rowScale);
     p.quantOut = reinterpret_cast<int8_t*>(DataPtr(output));
     p.quantScaleOut = reinterpret_cast<float*>(DataPtr(outputScale));
     ex->plan = gemm::MakePlan(p);
-    ex->workspaceBytes = ex->plan.workspaceBytes;
+    ex->SealWorkspace(ex->plan.workspaceBytes);
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;

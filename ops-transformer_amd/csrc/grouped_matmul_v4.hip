@@ -200,10 +200,7 @@ aclnnStatus PlanGroupedMatmul(
     const bool wTransposed = !nz && IsLastTwoDimsTransposed(wt);
     OPAPI_CHECK(nz || wTransposed || IsContiguous(wt), kInvalid,
                 "weight must be contiguous [E,K,N] or the transposed view of contiguous [E,N,K] storage");
-    OPAPI_CHECK(IsContiguous(xt) && IsContiguous(yt) && IsContiguous(groupListOptional), kInvalid,
-                "x, y and groupList must be contiguous");
-    OPAPI_CHECK(scale == nullptr || IsContiguous(scale), kInvalid, "scale must be contiguous");
-    OPAPI_CHECK(perToken == nullptr || IsContiguous(perToken), kInvalid, "perTokenScale must be contiguous");
+    OPAPI_CHECK(IsContiguous(yt), kInvalid, "y must be contiguous");  // the other tensors may be strided views
     const aclTensor* all[] = {xt, wt, yt, groupListOptional, scale, perToken};
     for (const aclTensor* t : all) {
         OPAPI_CHECK(t == nullptr || t->data != nullptr, ACLNN_ERR_PARAM_NULLPTR, "a tensor carries no device memory");
@@ -212,7 +209,7 @@ aclnnStatus PlanGroupedMatmul(
     auto* ex = new (std::nothrow) GroupedMatmulExecutor();
     OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
     gemm::Problem& p = ex->problem;
-    p.x = reinterpret_cast<const int8_t*>(DataPtr(xt));
+    OPAPI_BIND(ex, xt, &p.x);
     p.w = reinterpret_cast<const int8_t*>(DataPtr(wt));
     p.wKMajor = wTransposed;
     p.wNz = nz;
@@ -220,7 +217,7 @@ aclnnStatus PlanGroupedMatmul(
     p.K = k;
     p.N = n;
     p.groups = static_cast<int32_t>(groupListLen);
-    p.groupList = DataPtr(groupListOptional);
+    OPAPI_BIND(ex, groupListOptional, &p.groupList);
     p.groupListIsInt64 = groupListOptional->dtype == ACL_INT64;
     p.groupListKind = groupListType == 2 ? gemm::GroupListKind::kSparse
                       : groupListType == 1 ? gemm::GroupListKind::kCount : gemm::GroupListKind::kCumsum;
@@ -230,13 +227,13 @@ aclnnStatus PlanGroupedMatmul(
         p.epilogue = gemm::Epilogue::kInt32;
     } else {
         p.epilogue = gemm::Epilogue::kDequant;
-        p.scale = DataPtr(scale);
+        OPAPI_BIND(ex, scale, &p.scale);
         p.scaleDtype = static_cast<int>(scale->dtype);
-        p.rowScale = perToken != nullptr ? reinterpret_cast<const float*>(DataPtr(perToken)) : nullptr;
+        OPAPI_BIND(ex, perToken, &p.rowScale);
     }
     p.expectedRowsPerGroup = expectedRowsPerGroup;
     ex->plan = gemm::MakePlan(p);
-    ex->workspaceBytes = ex->plan.workspaceBytes;
+    ex->SealWorkspace(ex->plan.workspaceBytes);
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;

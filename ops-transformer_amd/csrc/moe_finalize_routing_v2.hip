@@ -271,7 +271,7 @@ extern "C" aclnnStatus aclnnMoeFinalizeRoutingV2GetWorkspaceSize(
                               expertIdxOptional, out};
     for (const aclTensor* t : all) {
         if (t == nullptr) continue;
-        OPAPI_CHECK(IsContiguous(t), kInvalid, "all tensors must be contiguous");
+        OPAPI_CHECK(t != out || IsContiguous(t), kInvalid, "out must be contiguous");  // inputs may be strided views
         OPAPI_CHECK(Numel(t) == 0 || t->data != nullptr, ACLNN_ERR_PARAM_NULLPTR, "a tensor carries no device memory");
     }
 
@@ -280,13 +280,13 @@ extern "C" aclnnStatus aclnnMoeFinalizeRoutingV2GetWorkspaceSize(
     ex->dtype = dt;
     ex->scaleIsF32 = (scalesOptional != nullptr && scalesOptional->dtype == ACL_FLOAT) ? 1 : 0;
     FinalizeArgs& a = ex->args;
-    a.expandedX = DataPtr(expandedX);
-    a.expandedRowIdx = reinterpret_cast<const int32_t*>(DataPtr(expandedRowIdx));
-    a.x1 = DataPtr(x1Optional);
-    a.x2 = DataPtr(x2Optional);
-    a.bias = DataPtr(biasOptional);
-    a.scales = DataPtr(scalesOptional);
-    a.expertIdx = reinterpret_cast<const int32_t*>(DataPtr(expertIdxOptional));
+    OPAPI_BIND(ex, expandedX, &a.expandedX);
+    OPAPI_BIND(ex, expandedRowIdx, &a.expandedRowIdx);
+    OPAPI_BIND(ex, x1Optional, &a.x1);
+    OPAPI_BIND(ex, x2Optional, &a.x2);
+    OPAPI_BIND(ex, biasOptional, &a.bias);
+    OPAPI_BIND(ex, scalesOptional, &a.scales);
+    OPAPI_BIND(ex, expertIdxOptional, &a.expertIdx);
     a.out = DataPtr(out);
     a.tokens = n;
     a.hidden = h;
@@ -298,8 +298,8 @@ extern "C" aclnnStatus aclnnMoeFinalizeRoutingV2GetWorkspaceSize(
                       reinterpret_cast<uintptr_t>(a.x1) | reinterpret_cast<uintptr_t>(a.x2) |
                       reinterpret_cast<uintptr_t>(a.bias);
     ex->vectorOk = (h % vec == 0) && (align % 16 == 0);
-    ex->workspaceBytes = 0;
-    *workspaceSize = 0;
+    ex->SealWorkspace(0);
+    *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;
 }

@@ -295,9 +295,8 @@ extern "C" aclnnStatus aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize(
         OPAPI_CHECK(IsContiguous(softmaxResultOutOptional), kInvalid, "softmaxResult must be contiguous");
     }
     OPAPI_CHECK(cols <= kMaxCols, kInvalid, "this build handles at most %lld experts per row", (long long)kMaxCols);
-    OPAPI_CHECK(IsContiguous(x) && IsContiguous(yOut) && IsContiguous(expertIdxOut) &&
-                    (finishedOptional == nullptr || IsContiguous(finishedOptional)), kInvalid,
-                "all tensors must be contiguous");
+    OPAPI_CHECK(IsContiguous(yOut) && IsContiguous(expertIdxOut), kInvalid,
+                "the outputs must be contiguous");  // x and finished may be strided views
     if (rows > 0) {
         OPAPI_CHECK(x->data != nullptr && yOut->data != nullptr && expertIdxOut->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
                     "x / yOut / expertIdxOut carry no device memory");
@@ -310,8 +309,8 @@ extern "C" aclnnStatus aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize(
     auto* ex = new (std::nothrow) GatingExecutor();
     OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
     ex->dtype = x->dtype;
-    ex->args.x = DataPtr(x);
-    ex->args.finished = reinterpret_cast<const uint8_t*>(DataPtr(finishedOptional));
+    OPAPI_BIND(ex, x, &ex->args.x);
+    OPAPI_BIND(ex, finishedOptional, &ex->args.finished);
     ex->args.y = DataPtr(yOut);
     ex->args.expertIdx = reinterpret_cast<int32_t*>(DataPtr(expertIdxOut));
     ex->args.softmaxOut = wantSoftmax ? reinterpret_cast<float*>(DataPtr(softmaxResultOutOptional)) : nullptr;
@@ -319,7 +318,8 @@ extern "C" aclnnStatus aclnnMoeGatingTopKSoftmaxV2GetWorkspaceSize(
     ex->args.cols = static_cast<int32_t>(cols);
     ex->args.k = static_cast<int32_t>(k);
     ex->args.renorm = static_cast<int32_t>(renorm);
-    *workspaceSize = 0;
+    ex->SealWorkspace(0);
+    *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;
 }

@@ -934,8 +934,8 @@ aclnnStatus PlanRoutingV2(const aclTensor* x, const aclTensor* expertIdx, const 
         aclnnStatus st = checkTokenCount(expertTokensBeforeCapacityOut, "expertTokensBeforeCapacity");
         if (st != ACLNN_SUCCESS) return st;
     }
-    OPAPI_CHECK(IsContiguous(x) && IsContiguous(expertIdx) && IsContiguous(expandedXOut) && IsContiguous(expandedRowIdxOut),
-                kInvalid, "x, expertIdx, expandedXOut and expandedRowIdxOut must be contiguous");
+    OPAPI_CHECK(IsContiguous(expandedXOut) && IsContiguous(expandedRowIdxOut), kInvalid,
+                "expandedXOut and expandedRowIdxOut must be contiguous");  // the inputs may be strided views
     if (total > 0) {
         OPAPI_CHECK(expertIdx->data != nullptr && expandedRowIdxOut->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
                     "expertIdx / expandedRowIdxOut carry no device memory");
@@ -961,8 +961,7 @@ aclnnStatus PlanRoutingV2(const aclTensor* x, const aclTensor* expertIdx, const 
             OPAPI_CHECK(scaleOptional->dims[0] == 1 || scaleOptional->dims[0] == expertNum, kInvalid,
                         "The first dim of scale should be 1 or expert_num.");
             OPAPI_CHECK(scaleOptional->dims[1] == cols, kInvalid, "The second dim of scale should be %lld.", (long long)cols);
-            OPAPI_CHECK(IsContiguous(scaleOptional) && (total == 0 || scaleOptional->data != nullptr), kInvalid,
-                        "scale must be contiguous device memory");
+            OPAPI_CHECK(total == 0 || scaleOptional->data != nullptr, ACLNN_ERR_PARAM_NULLPTR, "scale carries no device memory");
             smoothPerExpert = scaleOptional->dims[0] != 1;
         }
         OPAPI_CHECK(dynamicQuantScaleOut != nullptr, ACLNN_ERR_PARAM_NULLPTR, "DynamicQuantScale is nullptr!");
@@ -982,14 +981,14 @@ aclnnStatus PlanRoutingV2(const aclTensor* x, const aclTensor* expertIdx, const 
         ex->staticOffset = reinterpret_cast<const float*>(DataPtr(offsetOptional));
     } else if (quantMode == 1) {
         ex->dynamicQuant = true;
-        ex->scale = reinterpret_cast<const float*>(DataPtr(scaleOptional));
+        OPAPI_BIND(ex, scaleOptional, &ex->scale);
         ex->smoothPerExpert = smoothPerExpert;
         ex->expandedScale = reinterpret_cast<float*>(DataPtr(dynamicQuantScaleOut));
     }
     ex->xDtype = x->dtype;
     ex->cols = cols;
-    ex->x = DataPtr(x);
-    ex->expertIdx = reinterpret_cast<const int32_t*>(DataPtr(expertIdx));
+    OPAPI_BIND(ex, x, &ex->x);
+    OPAPI_BIND(ex, expertIdx, &ex->expertIdx);
     ex->expandedX = DataPtr(expandedXOut);
     ex->expandedRowIdx = reinterpret_cast<int32_t*>(DataPtr(expandedRowIdxOut));
     ex->countOrCumsum = countFlag != 0 ? reinterpret_cast<int32_t*>(DataPtr(expertTokensCountOrCumsumOut)) : nullptr;
@@ -1004,6 +1003,7 @@ aclnnStatus PlanRoutingV2(const aclTensor* x, const aclTensor* expertIdx, const 
     ex->dropPad = static_cast<int>(dropPadMode);
     ex->countFlag = static_cast<int>(countFlag);
     ex->Plan();
+    ex->SealWorkspace(ex->workspaceBytes);
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;
@@ -1129,8 +1129,7 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
                     "expandedScaleOut must not be null when scale is given or quant_mode is 1");
         OPAPI_CHECK(expandedScaleOut->dtype == ACL_FLOAT && expandedScaleOut->dims.size() == 1 &&
                         expandedScaleOut->dims[0] == total, kInvalid, "expandedScaleOut must be FLOAT [%lld]", (long long)total);
-        OPAPI_CHECK((scaleOptional == nullptr || IsContiguous(scaleOptional)) && IsContiguous(expandedScaleOut), kInvalid,
-                    "scale tensors must be contiguous");
+        OPAPI_CHECK(IsContiguous(expandedScaleOut), kInvalid, "expandedScaleOut must be contiguous");
     }
     if (dynamicQuant) OPAPI_CHECK(expandedXOut->dtype == ACL_INT8, kInvalid, "expandedXOut must be INT8 when quant_mode is 1");
     else OPAPI_CHECK(expandedXOut->dtype == x->dtype, kInvalid, "expandedXOut dtype must equal x dtype without quantisation");
@@ -1147,8 +1146,8 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
         OPAPI_CHECK(expertTokensCountOrCumsumOut->dims.size() == 1 && expertTokensCountOrCumsumOut->dims[0] == active,
                     kInvalid, "expertTokensCountOrCumsumOut must be [%lld]", (long long)active);
     }
-    OPAPI_CHECK(IsContiguous(x) && IsContiguous(expertIdx) && IsContiguous(expandedXOut) && IsContiguous(expandedRowIdxOut) &&
-                    IsContiguous(expertTokensCountOrCumsumOut), kInvalid, "all tensors must be contiguous");
+    OPAPI_CHECK(IsContiguous(expandedXOut) && IsContiguous(expandedRowIdxOut) && IsContiguous(expertTokensCountOrCumsumOut),
+                kInvalid, "the outputs must be contiguous");  // the inputs may be strided views
     OPAPI_CHECK(expertTokensCountOrCumsumOut->data != nullptr, ACLNN_ERR_PARAM_NULLPTR,
                 "expertTokensCountOrCumsumOut carries no device memory");
     if (total > 0) {
@@ -1165,8 +1164,8 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
     auto* ex = new (std::nothrow) InitRoutingExecutor();
     OPAPI_CHECK(ex != nullptr, ACLNN_ERR_INNER_CREATE_EXECUTOR, "out of host memory");
     ex->v3 = true;
-    ex->x = DataPtr(x);
-    ex->expertIdx = reinterpret_cast<const int32_t*>(DataPtr(expertIdx));
+    OPAPI_BIND(ex, x, &ex->x);
+    OPAPI_BIND(ex, expertIdx, &ex->expertIdx);
     ex->expandedX = DataPtr(expandedXOut);
     if (rowIdxType == 1) ex->expandedRowIdx = reinterpret_cast<int32_t*>(DataPtr(expandedRowIdxOut));
     else ex->gatherIdxOut = reinterpret_cast<int32_t*>(DataPtr(expandedRowIdxOut));
@@ -1174,7 +1173,7 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
     ex->countMode = static_cast<int>(expertTokensNumType);
     // key/value pairs written: min(active + 1, expertNum), as the reference sizes its copy-out
     ex->kvPairs = static_cast<int32_t>(active + 1 < expertNum ? active + 1 : expertNum);
-    ex->scale = scaleOptional != nullptr ? reinterpret_cast<const float*>(DataPtr(scaleOptional)) : nullptr;
+    OPAPI_BIND(ex, scaleOptional, &ex->scale);
     ex->expandedScale = (dynamicQuant || scaleOptional != nullptr) ? reinterpret_cast<float*>(DataPtr(expandedScaleOut)) : nullptr;
     ex->dynamicQuant = dynamicQuant;
     ex->xDtype = x->dtype;
@@ -1190,6 +1189,7 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
     ex->expertNum = active + (remap ? 1 : 0);  // key values the sort sees
     ex->countFlag = 2;                          // the sort emits plain int32 counts; CountV3Kernel shapes the output
     ex->Plan();
+    ex->SealWorkspace(ex->workspaceBytes);
     *workspaceSize = ex->workspaceBytes;
     *executor = ex;
     return ACLNN_SUCCESS;

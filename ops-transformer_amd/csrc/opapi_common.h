@@ -31,11 +31,49 @@ struct aclIntArray {
     std::vector<int64_t> values;
 };
 
+namespace opapi {
+// An input whose view is not contiguous is copied into the workspace (behind the operator's own part of it) at the
+// start of the second phase, as the reference makes such inputs contiguous before its kernels run
+// (gmm/grouped_matmul_swiglu_quant/op_host/op_api/aclnn_grouped_matmul_swiglu_quant.cpp:431-445).
+struct StagedInput {
+    void* slotAddr = nullptr;  // address of the executor's pointer field that the kernels read
+    uint64_t offset = 0;       // byte offset of the copy inside the staging area
+    const char* src = nullptr; // first element of the view
+    int64_t numel = 0;
+    int32_t nd = 0;
+    int32_t elemSize = 0;
+    int64_t dims[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int64_t strides[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // in elements
+};
+}  // namespace opapi
+
 struct aclOpExecutor {
-    uint64_t workspaceBytes = 0;
+    uint64_t workspaceBytes = 0;  // what the caller provides: the operator's own workspace, then the staging area
+    uint64_t stagingBase = 0;
+    uint64_t stagingBytes = 0;
+    std::vector<opapi::StagedInput> staged;
     virtual ~aclOpExecutor() = default;
     // Enqueue all kernels of the op on `stream`; must not synchronise with the host.
     virtual aclnnStatus Run(void* workspace, hipStream_t stream) = 0;
+
+    // Stores into *slot the pointer the kernels are to read input `t` through: its data when the view is contiguous
+    // (or absent, or empty), otherwise a 256-byte aligned stand-in that the second phase replaces by the address of a
+    // contiguous copy in the workspace.  Planning decisions that look at pointer alignment therefore hold for both.
+    template <typename T>
+    aclnnStatus Bind(const aclTensor* t, T** slot) {
+        const void* p = nullptr;
+        const aclnnStatus st = BindRaw(t, slot, &p);
+        *slot = static_cast<T*>(const_cast<void*>(p));
+        return st;
+    }
+    // Adds the staging area behind `ownBytes` of operator workspace and sets workspaceBytes.
+    void SealWorkspace(uint64_t ownBytes) {
+        stagingBase = (ownBytes + 255) / 256 * 256;
+        workspaceBytes = stagingBytes > 0 ? stagingBase + stagingBytes : ownBytes;
+    }
+
+   private:
+    aclnnStatus BindRaw(const aclTensor* t, void* slotAddr, const void** now);
 };
 
 namespace opapi {
@@ -140,6 +178,16 @@ class KernelTimer {
             OPAPI_CHECK(!::opapi::HasNegativeDim(opapiT_), ACLNN_ERR_PARAM_INVALID,                           \
                         "%s: a tensor has a negative extent: %s", __func__, ::opapi::ShapeStr(opapiT_).c_str()); \
         }                                                                                                     \
+    } while (0)
+
+// Binds input `t` to the executor's pointer field (see aclOpExecutor::Bind); on failure the executor is released.
+#define OPAPI_BIND(ex, t, slot)                             \
+    do {                                                    \
+        const aclnnStatus opapiBind_ = (ex)->Bind((t), (slot)); \
+        if (opapiBind_ != ACLNN_SUCCESS) {                  \
+            delete (ex);                                    \
+            return opapiBind_;                              \
+        }                                                   \
     } while (0)
 
 #define OPAPI_CHECK_NOTNULL(ptr, name) \

@@ -658,3 +658,31 @@ def test_negative_extents_are_rejected_everywhere(aclnn):
     for api, args in cases:
         code, msg = _status(aclnn, api, args)
         assert code == INVALID and "negative extent" in msg, (api, code, msg)
+
+
+# ------------------------------------------------------------------------------------------------ strided inputs
+def test_strided_inputs_are_staged_in_the_workspace(aclnn):
+    """A non-contiguous input costs a contiguous copy in the workspace (rounded up to 256 bytes); outputs must stay
+    contiguous; negative strides are refused."""
+    T_, K, H = 12, 2, 7
+    base = _fin_args(aclnn, T_=T_, K=K, H=H)
+    code, ws0 = _status(aclnn, "aclnnMoeFinalizeRoutingV2", base)
+    assert code == 0 and ws0 == 0
+    args = _fin_args(aclnn, T_=T_, K=K, H=H)
+    args[0] = T(aclnn, (T_ * K, H), F32, strides=[2 * H, 1]).h          # expandedX: every row twice as far apart
+    code, ws = _status(aclnn, "aclnnMoeFinalizeRoutingV2", args)
+    assert code == 0 and ws == (T_ * K * H * 4 + 255) // 256 * 256
+    args = _fin_args(aclnn, T_=T_, K=K, H=H)
+    args[-1] = T(aclnn, (T_, H), F32, strides=[2 * H, 1]).h             # out
+    code, msg = _status(aclnn, "aclnnMoeFinalizeRoutingV2", args)
+    assert code == INVALID and "out must be contiguous" in msg
+    args = _fin_args(aclnn, T_=T_, K=K, H=H)
+    args[0] = T(aclnn, (T_ * K, H), F32, strides=[H, -1]).h
+    code, msg = _status(aclnn, "aclnnMoeFinalizeRoutingV2", args)
+    assert code == INVALID and "negative strides" in msg
+
+    own = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=16, K=256, N=512, E=4))[1]
+    args = _swiglu_args(aclnn, M=16, K=256, N=512, E=4)
+    args[0] = T(aclnn, (16, 256), I8, strides=[512, 1]).h                # x
+    code, ws = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", args)
+    assert code == 0 and ws == (own + 255) // 256 * 256 + 16 * 256
