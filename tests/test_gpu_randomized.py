@@ -1,0 +1,164 @@
+"""Seeded random sweeps over shapes and modes, each case against the CPU oracle to the bar of its operator.  The
+parametrised tests elsewhere pick shapes by hand (tile boundaries, reference unit-test shapes); these draw them, so that
+combinations nobody thought of (odd widths with drop/pad, a one-expert range, K that leaves the fast kernel ...) get
+exercised too.  Sizes stay small: every case takes the oracle milliseconds."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+SEEDS = list(range(24))
+
+
+def _np(t):
+    return None if t is None else t.cpu().numpy()
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_routing_v2_random(aclnn, oracle, dev, seed):
+    rng = np.random.default_rng(1000 + seed)
+    T, K = int(rng.integers(1, 400)), int(rng.integers(1, 9))
+    E = int(rng.choice([1, 2, 7, 64, 256, 511, 512, 513, 1000, 2048]))
+    dtype = [np.int8, np.float16, np.float32][seed % 3]
+    H = int(rng.integers(1, 200)) if seed % 2 else int(rng.integers(1, 40)) * 16
+    x = rng.integers(-100, 100, (T, H)).astype(dtype)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    if seed % 4 == 3 and T >= 1:
+        C = int(rng.integers(1, T + 1))
+        kw = dict(expert_num=E, expert_capacity=C, drop_pad_mode=1, expert_tokens_before_capacity_flag=bool(seed % 8 == 3))
+        okw = dict(expert_num=E, expert_capacity=C, drop_pad_mode=1, before_capacity_flag=kw["expert_tokens_before_capacity_flag"])
+    else:
+        active = int(rng.integers(0, T * K + 5)) if seed % 3 == 0 else 0
+        flag = int(rng.integers(0, 3))
+        kw = dict(expert_num=E, active_num=active, expert_tokens_count_or_cumsum_flag=flag)
+        okw = dict(expert_num=E, active_num=active, count_flag=flag)
+    got = aclnn.moe_init_routing_v2(torch.from_numpy(x).to(dev), torch.from_numpy(idx).to(dev), **kw)
+    torch.cuda.synchronize()
+    want = oracle.moe_init_routing_v2(x, idx, **okw)
+    for g, w, name in zip(got, want, ("expandedX", "expandedRowIdx", "countOrCumsum", "beforeCapacity")):
+        assert (g is None) == (w is None), name
+        if g is not None:
+            assert np.array_equal(_np(g), w), (name, kw, T, K, E, H)
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_routing_v3_random(aclnn, oracle, dev, seed):
+    rng = np.random.default_rng(2000 + seed)
+    T, K = int(rng.integers(1, 400)), int(rng.integers(1, 9))
+    E = int(rng.choice([1, 3, 64, 256, 600, 2048, 5000]))
+    start = int(rng.integers(0, E))
+    end = int(rng.integers(start + 1, min(E, start + 2047) + 1))
+    rng_ = None if (seed % 3 == 0 and E <= 2048) else (start, end)
+    H = int(rng.integers(1, 30)) * 4
+    mode = seed % 3
+    row_idx_type = seed % 2
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    if seed % 4 == 1:                                      # dynamic quantisation
+        name = ["f32", "f16", "bf16"][seed % 3]
+        tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[name]
+        code = {"f32": oracle.DT_F32, "f16": oracle.DT_F16, "bf16": oracle.DT_BF16}[name]
+        xt = torch.from_numpy((rng.standard_normal((T, H)) * 2).astype(np.float32)).to(tdt)
+        bits = xt.numpy() if name == "f32" else xt.view(torch.int16).numpy().view(np.uint16)
+        n_active = (end - start) if rng_ is not None else E
+        smooth = (rng.random((n_active, H)) + 0.5).astype(np.float32) if seed % 8 == 1 else None
+        got = aclnn.moe_init_routing_v3(xt.to(dev), torch.from_numpy(idx).to(dev),
+                                        None if smooth is None else torch.from_numpy(smooth).to(dev), expert_num=E,
+                                        expert_tokens_num_type=mode, quant_mode=1, active_expert_range=rng_,
+                                        row_idx_type=row_idx_type)
+        torch.cuda.synchronize()
+        want = oracle.moe_init_routing_v3_quant(bits, idx, smooth, E, rng_, mode, row_idx_type, dtype=code)
+    else:
+        x = rng.integers(-100, 100, (T, H)).astype(np.int8)
+        scale = rng.random(T).astype(np.float32) if seed % 2 else None
+        got = aclnn.moe_init_routing_v3(torch.from_numpy(x).to(dev), torch.from_numpy(idx).to(dev),
+                                        None if scale is None else torch.from_numpy(scale).to(dev), expert_num=E,
+                                        expert_tokens_num_type=mode, active_expert_range=rng_, row_idx_type=row_idx_type)
+        torch.cuda.synchronize()
+        want = oracle.moe_init_routing_v3(x, idx, scale, E, rng_, mode, row_idx_type)
+    ex, ri, cnt, es = [_np(g) for g in got]
+    ex_r, ri_r, cnt_r, es_r = want
+    assert np.array_equal(cnt, cnt_r), (T, K, E, rng_, mode)
+    kept = int(((idx >= (rng_[0] if rng_ else 0)) & (idx < (rng_[1] if rng_ else E))).sum())
+    assert np.array_equal(ri, ri_r)
+    assert np.array_equal(ex[:kept], ex_r[:kept])          # rows behind the kept ones are not written
+    if es_r is not None:
+        assert np.array_equal(es[:kept], es_r[:kept])
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_grouped_gemm_random(aclnn, oracle, dev, seed):
+    rng = np.random.default_rng(3000 + seed)
+    M = int(rng.integers(1, 700))
+    K = int(rng.choice([16, 48, 128, 200, 256, 384, 1024]))
+    N = int(rng.choice([8, 64, 96, 256, 264, 512]))
+    E = int(rng.choice([1, 2, 5, 16, 40]))
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
+    # every fifth case leaves half of the rows behind the last group: they must stay untouched
+    sizes = rng.multinomial(M // 2 if seed % 5 == 4 else M, rng.dirichlet(np.ones(E) * 0.5))
+    cumsum = np.cumsum(sizes).astype(np.int64)
+    covered = int(cumsum[-1])
+    xd = torch.from_numpy(x).to(dev)
+    w_dev = torch.from_numpy(wt).to(dev)
+    wv = w_dev.transpose(1, 2) if seed % 3 else w_dev.transpose(1, 2).contiguous()
+    list_type = seed % 2
+    gl = cumsum if list_type == 0 else sizes.astype(np.int64)
+    gld = torch.from_numpy(gl).to(dev)
+    kw = dict(split_item=3, group_type=0, group_list_type=list_type)
+
+    ref = oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)
+    out = torch.full((M, N), -7, dtype=torch.int32, device=dev)
+    aclnn.grouped_matmul_v4([xd], [wv], group_list=gld, out=[out], **kw)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.array_equal(got[:covered], ref[:covered]) and (got[covered:] == -7).all(), (M, K, N, E, list_type)
+
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    per_token = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    ref = oracle.grouped_matmul_dequant(x, wt, scale, per_token, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
+    out = aclnn.grouped_matmul_v4([xd], [wv], scale=[torch.from_numpy(scale).to(dev)],
+                                  per_token_scale=[torch.from_numpy(per_token).to(dev)], group_list=gld,
+                                  output_dtype=torch.bfloat16, **kw)[0]
+    torch.cuda.synchronize()
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16)[:covered], ref[:covered])
+
+    if N % 2 == 0:
+        h_r, hs_r = oracle.grouped_matmul_swiglu_quant(x, wt, scale, per_token, cumsum, w_trans=True)
+        h, hs = aclnn.grouped_matmul_swiglu_quant(xd, wv, torch.from_numpy(cumsum).to(dev), torch.from_numpy(scale).to(dev),
+                                                  torch.from_numpy(per_token).to(dev))
+        torch.cuda.synchronize()
+        assert np.abs(h.cpu().numpy()[:covered].astype(np.int32) - h_r[:covered].astype(np.int32)).max(initial=0) <= 1
+        np.testing.assert_allclose(hs.cpu().numpy()[:covered], hs_r[:covered], rtol=1e-2)
+
+
+@pytest.mark.parametrize("seed", SEEDS[:12])
+def test_finalize_random(aclnn, oracle, dev, seed):
+    rng = np.random.default_rng(4000 + seed)
+    T, K, E = int(rng.integers(1, 200)), int(rng.integers(1, 9)), int(rng.integers(1, 40))
+    H = int(rng.integers(1, 300)) if seed % 2 else int(rng.integers(1, 60)) * 8
+    mode = [0, 2][seed % 2]
+    name = ["f32", "f16", "bf16"][seed % 3]
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[name]
+    code = {"f32": oracle.DT_F32, "f16": oracle.DT_F16, "bf16": oracle.DT_BF16}[name]
+
+    def make(shape):
+        t = torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(tdt)
+        return t, (t.numpy() if name == "f32" else t.view(torch.int16).numpy().view(np.uint16))
+
+    ex_t, ex_b = make((T * K, H))
+    x1_t, x1_b = make((T, H))
+    bias_t, bias_b = make((E, H))
+    sc_t, sc_b = make((T, K))
+    row_idx = rng.permutation(T * K).astype(np.int32)
+    eidx = rng.integers(0, E, (T, K)).astype(np.int32)
+    with_x1, with_bias = bool(seed % 3), bool(seed % 4)
+    got = aclnn.moe_finalize_routing_v2(ex_t.to(dev), torch.from_numpy(row_idx).to(dev), x1=x1_t.to(dev) if with_x1 else None,
+                                        bias=bias_t.to(dev) if with_bias else None, scales=sc_t.to(dev),
+                                        expert_idx=torch.from_numpy(eidx).to(dev) if with_bias else None, drop_pad_mode=mode)
+    torch.cuda.synchronize()
+    want = oracle.moe_finalize_routing_v2(ex_b, row_idx, x1_b if with_x1 else None, None, bias_b if with_bias else None, sc_b,
+                                          eidx if with_bias else None, drop_pad_mode=mode, dtype=code)
+    g = got.cpu()
+    g = g.numpy() if name == "f32" else g.view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(g, want), (T, K, E, H, mode, name)
