@@ -56,7 +56,6 @@ struct Problem {
 // Tile shape chosen from the static shape (M, groups); fixed for the lifetime of a plan.
 struct Plan {
     int tileM = 0;          // rows per workgroup tile (multiple of 32)
-    bool regPath = false;   // weights-in-registers kernel instead of the LDS ring kernel
     int wavesM = 1;         // 1 or 2 wave rows
     int subTilesM = 1;      // 32-row MFMA tiles per wave
     int64_t maxTiles = 0;   // launch bound on workgroups

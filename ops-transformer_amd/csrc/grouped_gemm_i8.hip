@@ -29,7 +29,6 @@
 
 #include <algorithm>
 #include <cstdlib>
-#include <string>
 #include <type_traits>
 
 #include "opapi_common.h"
@@ -792,401 +791,6 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     }
 }
 
-// ---------------------------------------------------------------------------------------------- fast path: weights in registers
-// Eight waves split the tile's 256 weight rows (output channels) 32 each and every wave covers all of the tile's
-// activation rows.  A wave's weight operands are then private to it, so they skip LDS altogether: each lane loads its
-// MFMA operand (16 bytes of one channel's k-slice) straight from global memory into registers, kDepth k-steps ahead.
-// Only the activations go through LDS (LDS-DMA ring of kDepth + 1 stages of 128 k-bytes).  Per CU this keeps
-// kDepth x 32 KB of weights in flight (192 KB at kDepth 6) instead of the one or two 32 KB stages an LDS ring has room
-// for, which is what it takes to stream weights at HBM speed with the MFMA work hidden underneath.
-//
-// The weight registers are not C++ variables.  The kernel is compiled with a VGPR budget that stops short of the top
-// 16 * kDepth registers (amdgpu_num_vgpr), and those registers are named literally in the inline assembly of the loads
-// and of the MFMAs, so the compiler can neither count the loads (its own s_waitcnt placement would treat the interleaved
-// LDS-DMA instructions as absent and wait for far more than the oldest stage) nor copy or spill a register whose load
-// is still pending.  Each k-step issues exactly kDmaPerWave DMA instructions and then 4 register loads per wave, so
-// "everything of the step issued kDepth steps ago has landed" is vmcnt <= (kDepth - 1) * (kDmaPerWave + 4).
-// The MFMAs are volatile assembly and stay in program order; the activation operands are double-buffered by hand
-// around them.
-template <int kSubM>
-struct RegCfg {
-    static constexpr int kWaves = 8;
-    static constexpr int kThreads = 64 * kWaves;
-    static constexpr int kTileM = 32 * kSubM;
-    static constexpr int kStageBytes = kTileM * 128;
-    static constexpr int kScratchBytes = (1 + kWaves) * kTileM * 4;
-    static constexpr int kStagesFit = (kLdsBudget - kScratchBytes) / kStageBytes;
-    static constexpr int kStages = kStagesFit > 9 ? 9 : kStagesFit;
-    static constexpr int kDepth = kStages - 1;
-    static constexpr int kLdsBytes = kStages * kStageBytes + kScratchBytes;
-    static constexpr int kBlocksA = kTileM / 8;  // DMA instructions (8 rows x 128 bytes) per activation stage
-    static constexpr int kDmaPerWave = (kBlocksA + kWaves - 1) / kWaves;
-    static constexpr int kLoadsPerStep = kDmaPerWave + 4;
-    static constexpr int kWeightReg0 = 256 - 16 * kDepth;  // first weight register; also the compiler's VGPR budget
-    static_assert(kDepth >= 2, "need at least two stages in flight");
-    static_assert((kDepth - 1) * kLoadsPerStep <= 63, "vmcnt is a 6-bit counter");
-};
-
-// 16 bytes per lane from (uniform base + lane offset + kOffset) into the fixed registers v[kReg : kReg + 3].
-template <int kReg, int kOffset>
-__device__ __forceinline__ void LoadFixed16(const char* uniformBase, uint32_t laneOffset) {
-    asm volatile("global_load_dwordx4 v[%3:%4], %0, %1 offset:%2"
-                 :: "v"(laneOffset), "s"(uniformBase), "n"(kOffset), "n"(kReg), "n"(kReg + 3) : "memory");
-}
-
-// acc += A (activation operand, compiler-allocated) x B (weight operand in the fixed registers v[kReg : kReg + 3]).
-template <int kReg>
-__device__ __forceinline__ void MfmaFixedB(v16i& acc, const v4i& av) {
-    asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, v[%2:%3], %0" : "+v"(acc) : "v"(av), "n"(kReg), "n"(kReg + 3));
-}
-
-// f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, kCount - 1>), in order.
-template <int kCount, typename F, int... kIs>
-__device__ __forceinline__ void StaticForImpl(F&& f, std::integer_sequence<int, kIs...>) {
-    (f(std::integral_constant<int, kIs>{}), ...);
-}
-template <int kCount, typename F>
-__device__ __forceinline__ void StaticFor(F&& f) {
-    StaticForImpl<kCount>(f, std::make_integer_sequence<int, kCount>{});
-}
-
-// Calls f(std::integral_constant<int, n>) for the n in 1..kMax that equals `active` (clamped into that range).
-template <int kMax, typename F>
-__device__ __forceinline__ void ForActive(int active, F& f) {
-    if constexpr (kMax == 1) {
-        f(std::integral_constant<int, 1>{});
-    } else {
-        if (active >= kMax) f(std::integral_constant<int, kMax>{});
-        else ForActive<kMax - 1>(active, f);
-    }
-}
-
-// Epilogue of one tile for the layout above.  acc[mi][v] is C[row, col] with row = 32*mi + 8*(v/4) + 4*lhi + (v%4) and
-// col = the wave's l32-th weight row: output channel colBase + 32*wave + l32, or for kSwiglu S column
-// colBase + 16*wave + (l32 % 16) with lanes 0..15 holding the activated half and lanes 16..31 the linear half.
-// Contains workgroup barriers: every wave must call it.
-template <int kSubM, Epilogue kEpi>
-__device__ __forceinline__ void RegTileEpilogue(const KernelArgs& a, const TileInfo& t, v16i (&acc)[kSubM], int wave,
-                                                int l32, int lhi, int tid, const float* ldsRowScale, float* ldsRowMax) {
-    constexpr int kTileM = 32 * kSubM;
-    const int32_t rows = t.rows, rowBase = t.rowBase, group = t.group;
-    // The row / address arithmetic below depends only on the lane, so the compiler would compute all of it once, keep
-    // some eighty values alive across the whole kernel and spill them; every reload in here then waits for all stores
-    // issued so far.  An opaque per-call zero folded into the lane index keeps the arithmetic inside the epilogue.
-    int opaqueZero;
-    asm volatile("v_mov_b32 %0, 0" : "=v"(opaqueZero));
-    lhi += opaqueZero;
-    l32 += opaqueZero;
-    if (kEpi == Epilogue::kInt32 || kEpi == Epilogue::kDequant) {
-        const bool hasRowScale = a.rowScale != nullptr;
-        const int32_t n = t.colBase + 32 * wave + l32;
-        const bool valid = n < a.N;
-        float sc = 0.0f;
-        if (kEpi == Epilogue::kDequant && valid) sc = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + n, a.scaleDtype);
-        // 16-bit outputs: neighbouring lanes hold neighbouring channels of the same rows.  They swap one value so that
-        // the even lane owns channels (c, c+1) of row r and the odd lane the same pair of row r+1: every lane stores one
-        // aligned 32-bit word.
-        const bool pairStores = kEpi == Epilogue::kDequant && a.outDtype != 0 && (a.N & 1) == 0 &&
-                                t.colBase + 32 * wave + 32 <= a.N;  // wave-uniform
-        const bool oddLane = (l32 & 1) != 0;
-#pragma unroll
-        for (int mi = 0; mi < kSubM; ++mi) {
-            if (32 * mi >= rows) continue;
-            if (kEpi == Epilogue::kInt32) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int r = 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
-                    if (r < rows && valid) static_cast<int32_t*>(a.out)[static_cast<int64_t>(rowBase + r) * a.N + n] = acc[mi][v];
-                }
-                continue;
-            }
-#pragma unroll
-            for (int p = 0; p < 8; ++p) {
-                const int r0 = 32 * mi + 8 * (p / 2) + 4 * lhi + 2 * (p % 2);  // row of v = 2p; v = 2p + 1 is the next row
-                float y0 = __fmul_rn(static_cast<float>(acc[mi][2 * p]), sc);
-                float y1 = __fmul_rn(static_cast<float>(acc[mi][2 * p + 1]), sc);
-                if (hasRowScale) {
-                    y0 = __fmul_rn(y0, ldsRowScale[r0 < rows ? r0 : 0]);
-                    y1 = __fmul_rn(y1, ldsRowScale[r0 + 1 < rows ? r0 + 1 : 0]);
-                }
-                const int64_t off0 = static_cast<int64_t>(rowBase + r0) * a.N + n;
-                if (a.outDtype == 0) {
-                    if (r0 < rows && valid) static_cast<float*>(a.out)[off0] = y0;
-                    if (r0 + 1 < rows && valid) static_cast<float*>(a.out)[off0 + a.N] = y1;
-                    continue;
-                }
-                uint32_t pk;  // both rows' values rounded to nearest even (low half = row r0)
-                if (a.outDtype == 27) {
-                    const Float2 f = {y0, y1};
-                    pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));  // v_cvt_pk_bf16_f32
-                } else {
-                    pk = static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y0))) |
-                         (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y1))) << 16);
-                }
-                if (pairStores) {
-                    // quad_perm [1,0,3,2]: exchange with the lane whose index differs in bit 0; the even lane keeps
-                    // (own row-r0 value, neighbour's row-r0 value), the odd lane (neighbour's row-r0+1 value, its own)
-                    const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
-                    const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
-                    const int r = oddLane ? r0 + 1 : r0;
-                    const int64_t off = static_cast<int64_t>(rowBase + r) * a.N + (oddLane ? n - 1 : n);
-                    if (r < rows) *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(a.out) + off) = word;
-                } else {
-                    if (r0 < rows && valid) static_cast<uint16_t*>(a.out)[off0] = static_cast<uint16_t>(pk & 0xffffu);
-                    if (r0 + 1 < rows && valid) static_cast<uint16_t*>(a.out)[off0 + a.N] = static_cast<uint16_t>(pk >> 16);
-                }
-            }
-        }
-    } else {
-        const int32_t j = t.colBase + 16 * wave + (l32 & 15);  // column of S
-        const bool jValid = j < a.halfN;
-        const int upper = l32 >> 4;  // after the swap below, lanes 16..31 of each half-wave work on the odd accumulators
-        float scA = 0.0f, scB = 0.0f;
-        if (jValid) {
-            scA = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + j, a.scaleDtype);
-            scB = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + a.halfN + j, a.scaleDtype);
-        }
-#pragma unroll
-        for (int mi = 0; mi < kSubM; ++mi) {
-            if (32 * mi >= rows) continue;  // workgroup-uniform
-#pragma unroll
-            for (int p = 0; p < 8; ++p) {
-                // v_permlane16_swap: rows of 16 lanes; the odd rows of the first operand trade places with the even rows
-                // of the second.  Before: lanes 0..15 hold the activated half and 16..31 the linear half, of row(2p) in
-                // the first operand and of row(2p+1) in the second.  After: every lane holds (activated, linear) of one
-                // element, lanes 0..15 for row(2p) and lanes 16..31 for row(2p+1).
-                typedef unsigned int Uint2 __attribute__((ext_vector_type(2)));
-                const Uint2 sw = __builtin_amdgcn_permlane16_swap(static_cast<unsigned int>(acc[mi][2 * p]),
-                                                                  static_cast<unsigned int>(acc[mi][2 * p + 1]), false, false);
-                const int v = 2 * p + upper;
-                const int r = 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
-                const bool ok = r < rows && jValid;
-                float s = 0.0f;
-                if (ok) {
-                    const float xs = ldsRowScale[r];
-                    const float ca = __fmul_rn(__fmul_rn(static_cast<float>(static_cast<int>(sw[0])), xs), scA);
-                    const float cb = __fmul_rn(__fmul_rn(static_cast<float>(static_cast<int>(sw[1])), xs), scB);
-                    // swish(ca) * cb with the hardware exp2 / reciprocal: a few ulp from the correctly rounded value,
-                    // far inside the +-1 LSB the int8 requantisation is held to
-                    s = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
-                    a.sOut[static_cast<int64_t>(rowBase + r) * a.halfN + j] = s;
-                }
-                // max |S| of this row over the wave's 16 columns
-                float m = fabsf(s);
-#pragma unroll
-                for (int d = 1; d < 16; d <<= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
-                if ((l32 & 15) == 0) ldsRowMax[wave * kTileM + r] = m;
-            }
-        }
-        __syncthreads();
-        // one partial maximum per (n-tile, row): no atomics and nothing to pre-zero; the requantisation folds them
-        if (tid < rows) {
-            float m = ldsRowMax[tid];
-#pragma unroll
-            for (int w = 1; w < 8; ++w) m = fmaxf(m, ldsRowMax[w * kTileM + tid]);
-            a.rowMax[static_cast<int64_t>(t.tileN) * a.M + rowBase + tid] = m;
-        }
-    }
-}
-
-// Persistent like StreamGemmKernel: one workgroup per CU, workgroup b serves XCD b % 8.
-template <int kSubM, Epilogue kEpi>
-__device__ __forceinline__ void RegStreamBody(const KernelArgs& a, const int32_t* __restrict__ sched) {
-    using Cfg = RegCfg<kSubM>;
-    asm volatile("" ::: "v255");  // the kernel owns all 256 VGPRs although the compiler allocates only the lower ones
-    constexpr int kTileM = Cfg::kTileM;
-    constexpr int kStages = Cfg::kStages;
-    constexpr int kDepth = Cfg::kDepth;
-    constexpr int kStageBytes = Cfg::kStageBytes;
-    constexpr bool kSwiglu = kEpi == Epilogue::kSwiglu;
-    extern __shared__ __attribute__((aligned(16))) char lds[];
-    float* const ldsRowScale = reinterpret_cast<float*>(lds + kStages * kStageBytes);  // [kTileM]
-    float* const ldsRowMax = ldsRowScale + kTileM;                                      // [8][kTileM]
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31;
-    const int lhi = lane >> 5;
-
-    const int64_t totalTiles = static_cast<int64_t>(sched[1]) * a.tilesN;
-    const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
-    const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
-    const int64_t slots = gridDim.x / kXcds;
-    auto decode = [&](int64_t local) { return DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, local); };
-
-    int64_t local = blockIdx.x / kXcds;
-    TileInfo cur = decode(local);
-    if (!cur.valid) return;
-    const int kSteps = a.K / 128;
-    // every tile takes a whole number of rounds of kDepth steps, so that a k-step always meets the same register set;
-    // the steps past kSteps only keep the load counts regular (they re-fetch the last k-slice and compute nothing)
-    const int stepsPerTile = (kSteps + kDepth - 1) / kDepth * kDepth;
-
-    // ---- issue side: always exactly one round (kDepth steps) ahead of the compute side, across tile boundaries ----
-    const char* issX = nullptr;
-    const char* issW = nullptr;
-    uint32_t aLaneOff[Cfg::kDmaPerWave];
-    uint32_t bLaneOff = 0;
-    auto setupIssue = [&](const TileInfo& iss) {
-        issX = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(iss.rowBase) * a.K;
-        issW = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(iss.group) * a.wGroupStride;
-        // activations: lane -> (row inside the 8-row block, LDS chunk slot); it fetches the chunk LdsOffset puts there
-        const int rowIn = lane >> 3;
-        const int slot = lane & 7;
-#pragma unroll
-        for (int q = 0; q < Cfg::kDmaPerWave; ++q) {
-            // blocks past the last one repeat it (same bytes to the same place) so that every wave issues the same
-            // number of DMAs; a block wholly past the tile's real rows reads a single chunk
-            const int j = min(wave + q * Cfg::kWaves, Cfg::kBlocksA - 1);
-            const int r = 8 * j + rowIn;
-            const int c = slot ^ ((r >> 1) & 7);
-            aLaneOff[q] = 8 * j >= iss.rows ? 0u : static_cast<uint32_t>(min(r, iss.rows - 1) * a.K + c * kChunk);
-        }
-        // weights: the lane's MFMA operand row (its output channel) and 16-byte k-slot
-        int32_t n;
-        if (kSwiglu) {
-            const int32_t jcol = min(iss.colBase + 16 * wave + (l32 & 15), a.halfN - 1);
-            n = l32 < 16 ? jcol : a.halfN + jcol;
-        } else {
-            n = min(iss.colBase + 32 * wave + l32, a.N - 1);
-        }
-        bLaneOff = static_cast<uint32_t>(n * a.K + lhi * kChunk);
-    };
-    const uint32_t ldsBase = LdsAddress(lds);
-    auto issueA = [&](int ringSlot, int step) {
-        const uint32_t dst = ldsBase + ringSlot * kStageBytes;
-        const char* const src = issX + min(step, kSteps - 1) * 128;
-#pragma unroll
-        for (int q = 0; q < Cfg::kDmaPerWave; ++q) {
-            const int j = min(wave + q * Cfg::kWaves, Cfg::kBlocksA - 1);
-            DmaToLdsAddr16(src, aLaneOff[q], dst + j * 1024);
-        }
-    };
-    // weight set d lives in v[kWeightReg0 + 16 d ...]: four operands of 16 bytes, one per 32-byte k-slice of the step
-    auto issueB = [&](auto dTag, int step) {
-        constexpr int kReg = Cfg::kWeightReg0 + 16 * decltype(dTag)::value;
-        const char* const src = UniformPtr(issW + min(step, kSteps - 1) * 128);
-        LoadFixed16<kReg + 0, 0>(src, bLaneOff);
-        LoadFixed16<kReg + 4, 32>(src, bLaneOff);
-        LoadFixed16<kReg + 8, 64>(src, bLaneOff);
-        LoadFixed16<kReg + 12, 96>(src, bLaneOff);
-    };
-
-    setupIssue(cur);
-    StaticFor<kDepth>([&](auto dTag) {
-        constexpr int d = decltype(dTag)::value;
-        issueA(d, d);
-        issueB(dTag, d);
-    });
-    int ring = 0;  // stage the compute side reads next; the issue side writes (ring + kDepth) % kStages
-
-    if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
-        ldsRowScale[tid] = a.rowScale[cur.rowBase + (tid < cur.rows ? tid : cur.rows - 1)];
-    }
-
-    // per-lane LDS offsets of the activation operand: row l32 of a 32-row block, chunk 2*ks + lhi
-    int aOff[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) aOff[ks] = LdsOffset<128>(l32, 2 * ks + lhi);
-    v16i acc[kSubM];
-    TileInfo following{};
-
-    // The k loop of one tile whose first kActive MFMA tiles hold real rows (the others are skipped entirely).
-    auto runTile = [&](auto activeTag) {
-        constexpr int kActive = decltype(activeTag)::value;
-#pragma unroll 1
-        for (int g = 0; g < stepsPerTile; g += kDepth) {
-            int issBase = g + kDepth;
-            if (issBase == stepsPerTile) {
-                // the round issued now is the first of this workgroup's next tile; past the last tile the current one
-                // is fetched again (nobody reads it), which keeps the number of outstanding loads per step constant
-                issBase = 0;
-                setupIssue(following.valid ? following : cur);
-            }
-            StaticFor<kDepth>([&](auto dTag) {
-                constexpr int d = decltype(dTag)::value;
-                constexpr int kReg = Cfg::kWeightReg0 + 16 * d;
-                // everything issued kDepth steps ago (this wave's share of activation stage `ring`, weight set d) is in
-                WaitVmcnt<(kDepth - 1) * Cfg::kLoadsPerStep>();
-                __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
-                issueA(ring == 0 ? kStages - 1 : ring - 1, issBase + d);
-                if (g + d < kSteps) {
-                    const char* const A = lds + ring * kStageBytes;
-                    // the MFMAs are volatile assembly (ordered as written, and LDS reads do not move across them): the
-                    // activation operands of k-slice ks + 1 are read before the MFMAs of k-slice ks are issued
-                    v4i av[2][kActive];
-#pragma unroll
-                    for (int mi = 0; mi < kActive; ++mi) av[0][mi] = *reinterpret_cast<const v4i*>(A + mi * 4096 + aOff[0]);
-                    StaticFor<4>([&](auto ksTag) {
-                        constexpr int ks = decltype(ksTag)::value;
-                        if (ks < 3) {
-#pragma unroll
-                            for (int mi = 0; mi < kActive; ++mi) {
-                                av[(ks + 1) & 1][mi] = *reinterpret_cast<const v4i*>(A + mi * 4096 + aOff[ks < 3 ? ks + 1 : 3]);
-                            }
-                        }
-#pragma unroll
-                        for (int mi = 0; mi < kActive; ++mi) MfmaFixedB<kReg + 4 * ks>(acc[mi], av[ks & 1][mi]);
-                    });
-                }
-                issueB(dTag, issBase + d);
-                ring = ring + 1 == kStages ? 0 : ring + 1;
-            });
-        }
-        // A matrix-core result may not be read by a vector instruction for 18 cycles after issue; the compiler cannot
-        // see the MFMAs inside the assembly, so the gap is made explicit, and every later use of an accumulator is made
-        // to depend on it.
-        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc[0]));
-#pragma unroll
-        for (int mi = 1; mi < kSubM; ++mi) asm volatile("" : "+v"(acc[mi]));
-    };
-
-    while (true) {
-        following = decode(local + slots);
-        // the next tile's per-row scale travels in a register until this tile's epilogue has read the LDS copy
-        float followingRowScale = 0.0f;
-        if (following.valid && kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
-            followingRowScale = a.rowScale[following.rowBase + (tid < following.rows ? tid : following.rows - 1)];
-        }
-#pragma unroll
-        for (int mi = 0; mi < kSubM; ++mi)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mi][v] = 0;
-
-        const int active = (cur.rows + 31) >> 5;  // 1..kSubM, workgroup-uniform
-        ForActive<kSubM>(active, runTile);
-
-        RegTileEpilogue<kSubM, kEpi>(a, cur, acc, wave, l32, lhi, tid, ldsRowScale, ldsRowMax);
-        // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
-        // stores and the loads in flight, which had the whole epilogue to land) before counting loads again.
-        WaitVmcnt<0>();
-        if (!following.valid) break;
-        __syncthreads();  // the epilogue's reads of ldsRowScale / ldsRowMax are done
-        if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) ldsRowScale[tid] = followingRowScale;
-        cur = following;
-        local += slots;
-    }
-}
-
-// __global__ wrappers: amdgpu_num_vgpr takes a literal, so each tile height gets its own (checked against RegCfg).  On
-// this target the attribute counts in units of two registers (it budgets the unified VGPR + AGPR file and no AGPRs are
-// used here), so HALF = first weight register / 2.
-#define OPAPI_REG_KERNEL(SUB, HALF)                                                                               \
-    template <Epilogue kEpi>                                                                                      \
-    __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(HALF))) void RegStreamGemmKernel##SUB(       \
-        KernelArgs a, const int32_t* __restrict__ sched) {                                                        \
-        static_assert(RegCfg<SUB>::kWeightReg0 == 2 * HALF, "VGPR budget must end where the weight registers begin"); \
-        RegStreamBody<SUB, kEpi>(a, sched);                                                                       \
-    }
-OPAPI_REG_KERNEL(1, 64)
-OPAPI_REG_KERNEL(2, 64)
-OPAPI_REG_KERNEL(3, 64)
-OPAPI_REG_KERNEL(4, 64)
-OPAPI_REG_KERNEL(5, 80)
-OPAPI_REG_KERNEL(6, 88)
-#undef OPAPI_REG_KERNEL
-
 // ---------------------------------------------------------------------------------------------- generic path
 constexpr int kGenStep = 128;  // k-bytes per step
 
@@ -1379,45 +983,9 @@ hipError_t LaunchStreamShape(const Plan& plan, const KernelArgs& args, const int
                     : LaunchStreamShapeOf<kEpi, false>(plan, args, sched, stream);
 }
 
-template <int kSubM, void (*kKernel)(KernelArgs, const int32_t*)>
-hipError_t LaunchReg(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
-    using Cfg = RegCfg<kSubM>;
-    const auto kernel = kKernel;
-    // the kernel is a template argument: one instantiation of this function, hence one static, per kernel
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
-    if (attr != hipSuccess) return attr;
-    int64_t grid = DeviceCuCount();
-    if (grid > maxTiles) grid = maxTiles;
-    grid = grid / kXcds * kXcds;
-    if (grid < kXcds) grid = kXcds;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, args, sched);
-    return hipGetLastError();
-}
-
-template <Epilogue kEpi>
-hipError_t LaunchRegShape(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
-    switch (plan.tileM) {
-        case 32: return LaunchReg<1, RegStreamGemmKernel1<kEpi>>(args, sched, plan.maxTiles, stream);
-        case 64: return LaunchReg<2, RegStreamGemmKernel2<kEpi>>(args, sched, plan.maxTiles, stream);
-        case 96: return LaunchReg<3, RegStreamGemmKernel3<kEpi>>(args, sched, plan.maxTiles, stream);
-        case 128: return LaunchReg<4, RegStreamGemmKernel4<kEpi>>(args, sched, plan.maxTiles, stream);
-        case 160: return LaunchReg<5, RegStreamGemmKernel5<kEpi>>(args, sched, plan.maxTiles, stream);
-        case 192: return LaunchReg<6, RegStreamGemmKernel6<kEpi>>(args, sched, plan.maxTiles, stream);
-        default: return hipErrorInvalidValue;  // 256-row tiles are served by the ring kernel
-    }
-}
-
-// Which fast kernel serves a plan.  The LDS ring kernel is the default: on the DeepSeek-V3 prefill shape it runs the
-// gate/up GEMM in 1.74 ms against 1.98 ms for the weights-in-registers kernel, whose 32-byte-granular weight loads cost
-// four L1 tag look-ups per cache line.  OPAPI_GEMM_PATH=reg selects the register kernel for tiles up to 192 rows (its
-// 256-row instantiation is not built: every wave re-reading all activation rows from LDS is a loss on MFMA-bound shapes).
-bool UseRegPath(const Plan& plan) { return plan.regPath; }
-
 template <Epilogue kEpi>
 hipError_t LaunchFast(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
-    return UseRegPath(plan) ? LaunchRegShape<kEpi>(plan, args, sched, stream)
-                            : LaunchStreamShape<kEpi>(plan, args, sched, stream);
+    return LaunchStreamShape<kEpi>(plan, args, sched, stream);
 }
 
 template <Epilogue kEpi>
@@ -1463,12 +1031,6 @@ Plan MakePlan(const Problem& p) {
         }
     } else {
         plan.tileM = want <= 32.0 ? 32 : 128;
-    }
-    {
-        // read at plan time (not cached) so that one process can plan either way
-        const char* env = std::getenv("OPAPI_GEMM_PATH");
-        plan.regPath = StreamOk(p) && !p.wNz && plan.tileM <= 192 && p.combineIndex == nullptr && env != nullptr &&
-                       std::string(env) == "reg";
     }
     plan.wavesM = plan.tileM >= 64 && StreamOk(p) ? 2 : 1;
     plan.subTilesM = (plan.tileM / 32 + plan.wavesM - 1) / plan.wavesM;

@@ -175,47 +175,6 @@ def test_v5_tuning_hint_changes_tiling_not_results(aclnn, oracle, dev, hint):
     assert np.array_equal(out.cpu().numpy(), ref)
 
 
-@pytest.fixture
-def reg_path(monkeypatch):
-    """Plans made inside the test use the weights-in-registers GEMM kernel (opt-in; the LDS ring kernel is the default)."""
-    monkeypatch.setenv("OPAPI_GEMM_PATH", "reg")
-
-
-@pytest.mark.parametrize("M,K,N,E,mode", [(37, 128, 24, 4, "ragged"), (512, 1024, 512, 8, "even"),
-                                          (1500, 384, 256, 10, "ragged"), (2048, 2048, 256, 16, "even"),
-                                          (640, 256, 256, 64, "sparse")])
-def test_register_kernel_int32_bit_exact(aclnn, oracle, dev, reg_path, M, K, N, E, mode):
-    rng = np.random.default_rng(M + K + N + 1)
-    x, wt, cumsum = _problem(rng, M, K, N, E, mode)
-    ref = oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)
-    out = torch.full((M, N), -7, dtype=torch.int32, device=dev)
-    aclnn.grouped_matmul_v4([torch.from_numpy(x).to(dev)], [_weight_views(wt, dev, "kmajor")],
-                            group_list=torch.from_numpy(cumsum).to(dev), split_item=3, group_type=0, out=[out])
-    torch.cuda.synchronize()
-    assert np.array_equal(out.cpu().numpy(), ref)
-
-
-def test_register_kernel_epilogues(aclnn, oracle, dev, reg_path):
-    """Down-projection (bf16, bit-exact) and SwiGLU-quant (+-1 LSB) epilogues of the register kernel."""
-    rng = np.random.default_rng(77)
-    M, K, N, E = 600, 1024, 520, 5
-    x, wt, cumsum = _problem(rng, M, K, N, E)
-    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
-    per_token = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
-    ref = oracle.grouped_matmul_dequant(x, wt, scale, per_token, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
-    xd, wv, gl = torch.from_numpy(x).to(dev), _weight_views(wt, dev, "kmajor"), torch.from_numpy(cumsum).to(dev)
-    out = aclnn.grouped_matmul_v4([xd], [wv], scale=[torch.from_numpy(scale).to(dev)],
-                                  per_token_scale=[torch.from_numpy(per_token).to(dev)], group_list=gl, split_item=3,
-                                  group_type=0, output_dtype=torch.bfloat16)[0]
-    torch.cuda.synchronize()
-    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), ref)
-    q_ref, s_ref = oracle.grouped_matmul_swiglu_quant(x, wt, scale, per_token, cumsum, w_trans=True)
-    q, qs = aclnn.grouped_matmul_swiglu_quant(xd, wv, gl, torch.from_numpy(scale).to(dev), torch.from_numpy(per_token).to(dev))
-    torch.cuda.synchronize()
-    assert np.abs(q.cpu().numpy().astype(np.int32) - q_ref.astype(np.int32)).max() <= 1
-    np.testing.assert_allclose(qs.cpu().numpy(), s_ref, rtol=1e-2)
-
-
 # ------------------------------------------------------------------------------------------------ sparse group lists
 @pytest.mark.parametrize("M,K,N,E,order", [(300, 256, 256, 16, "ascending"), (640, 512, 520, 64, "ascending"),
                                           (200, 128, 128, 8, "shuffled"), (96, 128, 72, 4, "all")])
