@@ -16,11 +16,11 @@
 // XCD's L2); inside a group, bands of 4 m-tiles walk the n-tiles together so weight columns are reused from L2.
 //
 // Two kernels share the tile decode and the epilogue:
-//   StreamGemmKernel  the fast path (K-contiguous weights, K a multiple of 128).  Persistent workgroups; operands go
+//   StreamGemmKernel  the fast path (K a multiple of 128; K-contiguous, blocked or row-major [K, N] weights).  Persistent workgroups; operands go
 //                     global -> LDS with global_load_lds_dwordx4 into a ring of 3..8 stages of 128 (or 64) k-bytes, so several
 //                     stages of weights are in flight per CU with no staging registers, and the ring keeps filling
 //                     with the next tile's first steps while the current tile's epilogue runs.
-//   GenericGemmKernel byte-wise loader for row-major [K, N] weights and for K not a multiple of 128: correct, slow.
+//   GenericGemmKernel byte-wise loader for K not a multiple of 128 and channel counts off the 16-byte grid: correct, slow.
 // LDS rows are XOR-swizzled in 16-byte chunks so that the 16 lanes the LDS serves per clock (64 banks) never collide,
 // for the DMA writes as well as for the MFMA operand reads.
 #include "grouped_gemm_i8.h"
@@ -583,10 +583,17 @@ __device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leavi
 // operand (16 consecutive k of one channel per lane) is read back with the transposing LDS load ds_read_b64_tr_b8:
 // per 16 lanes, lanes 2r and 2r + 1 supply the two 8-byte halves of row r (r = 0..7) and lane i receives column i,
 // i.e. with rows = 8 consecutive k and columns = 16 channels each lane gets 8 consecutive k of its channel.
-template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz>
+//
+// kNMajor: the weights are row-major [K, N] per expert (N contiguous), the reference's plain ND layout of the grouped
+// matmul.  A stage's weight part is then 128 k-rows of the tile's 256 channel bytes (one 256-byte run per k-row, two of
+// 128 bytes for the gate and up halves of a SwiGLU tile); it lies in LDS as [k][256] with the 16-byte chunks of row k
+// XOR-ed by k & 15, and the operands come out through the same transposing load as for the blocked layout (8
+// consecutive k-rows then sit in 8 different bank groups).
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor = false>
 __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     KernelArgs a, const int32_t* __restrict__ sched) {
-    static_assert(!kNz || kStep == 128, "the blocked weight layout is built for 128-byte k-steps");
+    static_assert(!(kNz || kNMajor) || kStep == 128, "the blocked and row-major weight layouts are built for 128-byte k-steps");
+    static_assert(!(kNz && kNMajor), "one weight layout at a time");
     using Cfg = StreamCfg<kSub0, kSub1, kStep>;
     constexpr int kSubM = kSub0;  // accumulator tiles per wave (wave row 1 uses the first kSub1 of them)
     constexpr int kTileM = Cfg::kTileM;
@@ -644,6 +651,20 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                 const int c = (LdsOffset<kStep>(r, slot) >> 4) % Cfg::kChunksPerRow;
                 const bool wholeInstrPast = Cfg::kRowsPerInstr * j >= iss.rows;
                 laneOff[q] = wholeInstrPast ? 0u : static_cast<uint32_t>(min(r, iss.rows - 1) * a.K + c * kChunk);
+            } else if (kNMajor) {
+                // weight instruction jw moves k-rows 4 * jw .. + 3 of the stage, 256 channel bytes each; lane ->
+                // (k-row lane / 16, LDS chunk slot lane % 16), fetching the logical chunk that the swizzle puts there.
+                // Chunks past the last channel are never stored: such lanes re-read the last real chunk.
+                const int jw = j - Cfg::kInstrA;
+                const int k = 4 * jw + lane / 16;
+                const int c = (lane % 16) ^ (k & 15);
+                int32_t col;
+                if (kSwiglu) {
+                    col = c < 8 ? min(iss.colBase + 16 * c, a.halfN - 16) : min(a.halfN + iss.colBase + 16 * (c - 8), a.N - 16);
+                } else {
+                    col = min(iss.colBase + 16 * c, a.N - 16);
+                }
+                laneOff[q] = static_cast<uint32_t>(k * a.N + col);
             } else if (kNz) {
                 // weight instruction jw moves 32 k-rows (x 32 channel bytes) of channel block jw / 4: 1 KB, contiguous
                 // in memory and in LDS; lane -> (k-row lane / 2, 16-byte half lane % 2)
@@ -660,7 +681,8 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     auto issueStage = [&](int ring) {
         const uint32_t dst = ldsBase + ring * kStageBytes;
         const int kOff = issStep * kStep;
-        const int kOffW = kNz ? kOff * 32 : kOff;  // blocked layout: one k is 32 bytes further
+        // blocked layout: one k is 32 bytes further; row-major: N bytes
+        const int kOffW = kNz ? kOff * 32 : (kNMajor ? kOff * a.N : kOff);
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
             const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
@@ -725,7 +747,22 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             auto loadSlice = [&](int ks, int buf) {
                 if (kMy == 0) return;
                 const int chunk = 2 * ks + lhi;
-                if constexpr (kNz) {
+                if constexpr (kNMajor) {
+                    // 16-lane group g: channels 16 * (g % 2) .. + 15 of the 32-channel block, k-half g / 2 (= lhi) of the
+                    // slice; lane j of the group supplies bytes (k = kBase + j / 2, channels 8 * (j % 2) .. + 7)
+                    const int j = lane & 15;
+                    const int k = 32 * ks + 16 * lhi + (j >> 1);
+                    const uint32_t bBase = ldsBase + ring * kStageBytes + kTileM * kStep + 8 * (j & 1);
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni) {
+                        const int c = (bRow0 + ni * bRowStep + 16 * ((lane >> 4) & 1)) >> 4;  // logical 16-byte chunk of the row
+                        const uint32_t lo = bBase + k * 256 + ((c ^ (k & 15)) << 4);
+                        const uint32_t hi = bBase + (k + 8) * 256 + ((c ^ ((k + 8) & 15)) << 4);
+                        const v2i vlo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(lo));
+                        const v2i vhi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(hi));
+                        bf[buf][ni] = v4i{vlo[0], vlo[1], vhi[0], vhi[1]};
+                    }
+                } else if constexpr (kNz) {
                     // 16-lane group g: channels 16 * (g % 2) .. + 15 of the block, k-half g / 2 (= lhi) of the slice;
                     // lane j of the group supplies bytes (k = kBase + j / 2, channels 8 * (j % 2) .. + 7)
                     const int j = lane & 15;
@@ -946,10 +983,10 @@ int DeviceCuCount() {
     return count;
 }
 
-template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz>
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor>
 hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
     using Cfg = StreamCfg<kSub0, kSub1, kStep>;
-    auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi, kNz>;
+    auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi, kNz, kNMajor>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
     if (attr != hipSuccess) return attr;
@@ -964,23 +1001,24 @@ hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t ma
 
 // Tile heights and their (wave row 0, wave row 1, k-step) shapes.  128-byte steps with a ring of three or more stages
 // stream best; 192 and 256 rows only leave room for two such stages.
-template <Epilogue kEpi, bool kNz>
+template <Epilogue kEpi, bool kNz, bool kNMajor>
 hipError_t LaunchStreamShapeOf(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
     switch (plan.tileM) {
-        case 32: return LaunchStream<1, 0, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
-        case 64: return LaunchStream<1, 1, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
-        case 96: return LaunchStream<2, 1, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
-        case 128: return LaunchStream<2, 2, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
-        case 160: return LaunchStream<3, 2, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
-        case 192: return LaunchStream<3, 3, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
-        default: return LaunchStream<4, 4, 128, kEpi, kNz>(args, sched, plan.maxTiles, stream);
+        case 32: return LaunchStream<1, 0, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        case 64: return LaunchStream<1, 1, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        case 96: return LaunchStream<2, 1, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        case 128: return LaunchStream<2, 2, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        case 160: return LaunchStream<3, 2, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        case 192: return LaunchStream<3, 3, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        default: return LaunchStream<4, 4, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
     }
 }
 
 template <Epilogue kEpi>
 hipError_t LaunchStreamShape(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
-    return args.wNz ? LaunchStreamShapeOf<kEpi, true>(plan, args, sched, stream)
-                    : LaunchStreamShapeOf<kEpi, false>(plan, args, sched, stream);
+    if (args.wNz) return LaunchStreamShapeOf<kEpi, true, false>(plan, args, sched, stream);
+    if (args.wStrideN == 1) return LaunchStreamShapeOf<kEpi, false, true>(plan, args, sched, stream);  // row-major [K, N]
+    return LaunchStreamShapeOf<kEpi, false, false>(plan, args, sched, stream);
 }
 
 template <Epilogue kEpi>
@@ -996,10 +1034,13 @@ hipError_t LaunchGenericShape(const Plan& plan, const KernelArgs& args, const in
     return hipGetLastError();
 }
 
-// The DMA ring needs K-contiguous weights, whole 128-byte k steps, 16-byte aligned bases and 32-bit offsets inside one
-// expert's weights.
+// The DMA ring needs whole 128-byte k steps, 16-byte aligned bases, 32-bit offsets inside one expert's weights and one of
+// the three weight layouts it knows: K-contiguous rows per channel, the blocked layout, or row-major [K, N].
 bool StreamOk(const Problem& p) {
-    const bool layoutOk = p.wNz ? (p.N % 32 == 0 && (p.epilogue != Epilogue::kSwiglu || (p.N / 2) % 32 == 0)) : p.wKMajor;
+    // blocked: whole 32-channel blocks; row-major: whole 16-byte chunks (per half of a SwiGLU tile)
+    const int64_t grain = p.wNz ? 32 : 16;
+    const bool layoutOk = p.wKMajor && !p.wNz ? true
+                          : (p.N % grain == 0 && (p.epilogue != Epilogue::kSwiglu || (p.N / 2) % grain == 0));
     return layoutOk && p.K % 128 == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
            reinterpret_cast<uintptr_t>(p.w) % kChunk == 0 && p.N * p.K < (1ll << 31);
 }

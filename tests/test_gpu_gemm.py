@@ -48,6 +48,13 @@ INT32_CASES = [  # M, K, N, E, mode, layout
     (300, 208, 72, 4, "ragged", "nd"),           # row-major [E,K,N] weight: byte-wise loader
     (100, 7168, 64, 2, "even", "kmajor"),        # |acc| beyond 2^24
     (640, 256, 256, 64, "sparse", "kmajor"),
+    # row-major [E, K, N] weights (the reference's plain ND layout) on the fast kernel: K % 128 == 0, N % 16 == 0
+    (37, 128, 16, 4, "ragged", "nd"),
+    (512, 1024, 512, 8, "even", "nd"),
+    (700, 512, 528, 3, "ragged", "nd"),          # tile 256; 528 = 2 * 256 + 16 channels: the last tile holds one chunk
+    (1500, 384, 256, 10, "ragged", "nd"),
+    (512, 4096, 256, 128, "ragged", "nd"),       # decode-like
+    (640, 256, 272, 64, "sparse", "nd"),
 ]
 
 
@@ -99,12 +106,13 @@ def test_down_projection_epilogue(aclnn, oracle, dev, M, K, N, E, scale_dtype, o
         scale_arg, sd = scale, oracle.DT_F32
     od = oracle.DT_BF16 if out_dtype == torch.bfloat16 else oracle.DT_F16
     ref = oracle.grouped_matmul_dequant(x, wt, scale_arg, per_token, cumsum, w_trans=True, scale_dtype=sd, out_dtype=od)
-    out = aclnn.grouped_matmul_v4([torch.from_numpy(x).to(dev)], [_weight_views(wt, dev, "kmajor")], scale=[scale_t],
-                                  per_token_scale=[torch.from_numpy(per_token).to(dev)],
-                                  group_list=torch.from_numpy(cumsum).to(dev), split_item=3, group_type=0,
-                                  output_dtype=out_dtype)[0]
-    torch.cuda.synchronize()
-    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+    for layout in ("kmajor", "nd"):       # K-contiguous storage behind a transposed view, and row-major [E, K, N]
+        out = aclnn.grouped_matmul_v4([torch.from_numpy(x).to(dev)], [_weight_views(wt, dev, layout)], scale=[scale_t],
+                                      per_token_scale=[torch.from_numpy(per_token).to(dev)],
+                                      group_list=torch.from_numpy(cumsum).to(dev), split_item=3, group_type=0,
+                                      output_dtype=out_dtype)[0]
+        torch.cuda.synchronize()
+        assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), ref), layout
 
 
 SWIGLU_CASES = [  # M, K, N, E, mode, layout, scale dtype
@@ -115,6 +123,9 @@ SWIGLU_CASES = [  # M, K, N, E, mode, layout, scale dtype
     (300, 512, 208, 5, "ragged", "kmajor", "bf16"),   # N/2 not a multiple of the tile
     (300, 512, 208, 5, "ragged", "kmajor", "f16"),
     (100, 200, 96, 3, "ragged", "nd", "f32"),
+    (512, 1024, 2048, 8, "ragged", "nd", "f32"),      # row-major weights on the fast kernel
+    (300, 512, 224, 5, "ragged", "nd", "bf16"),       # N/2 = 112 = 7 chunks: both halves of the tile are clamped
+    (512, 4096, 3072, 128, "ragged", "nd", "f32"),
 ]
 
 
