@@ -162,7 +162,9 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
         if (t == a.groups - 1) {
             tilePrefix[a.groups] = tileInc;
             a.sched[0] = covered;
-            a.sched[1] = tileInc;
+            // A well-formed list never needs more than maxMTiles m-tiles (M / tileM + groups).  A malformed one whose
+            // groups overlap could: the tiles beyond the table are dropped, so no kernel indexes past it.
+            a.sched[1] = tileInc < a.maxMTiles ? tileInc : a.maxMTiles;
         }
     }
     // group of every m-tile: scan[] still holds the inclusive m-tile prefix (zero-tile groups repeat their

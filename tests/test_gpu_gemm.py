@@ -87,6 +87,26 @@ def test_rows_beyond_last_group_untouched(aclnn, oracle, dev):
     assert np.array_equal(got[:120], ref[:120]) and (got[120:] == -7).all()
 
 
+@pytest.mark.parametrize("kind,values", [
+    ("cumsum", [300, 0, 300, 0, 300]),          # groups 0, 2 and 4 each claim every row: three times the tiles of a sane list
+    ("cumsum", [120, 50, 400, -7, 90]),         # not monotonic, beyond M, negative
+    ("count", [300, 300, 300, 300, 300]),       # counts add up to five times M
+    ("count", [-5, 400, 10, 0, 2000000000]),
+])
+def test_malformed_group_lists_stay_in_bounds(aclnn, dev, kind, values):
+    """A list that is not a cumsum / count list of M rows gives unspecified rows, but never an access outside the
+    tensors: boundaries are clamped into [0, M] and the tile table is cut at the size planned for a well-formed list."""
+    rng = np.random.default_rng(9)
+    M, K, N, E = 300, 128, 64, 5
+    x, wt, _ = _problem(rng, M, K, N, E, "even")
+    guard = torch.full((M + 64, N), -7, dtype=torch.int32, device=dev)
+    aclnn.grouped_matmul_v4([torch.from_numpy(x).to(dev)], [_weight_views(wt, dev, "kmajor")],
+                            group_list=torch.tensor(values, dtype=torch.int64, device=dev), split_item=3, group_type=0,
+                            group_list_type=0 if kind == "cumsum" else 1, out=[guard[:M]])
+    torch.cuda.synchronize()
+    assert (guard[M:] == -7).all()
+
+
 DEQUANT_CASES = [(64, 256, 128, 4, "f32", torch.bfloat16), (64, 256, 128, 4, "bf16", torch.bfloat16),
                  (64, 256, 128, 4, "f32", torch.float16), (512, 1024, 1024, 8, "f32", torch.bfloat16),
                  (333, 1536, 520, 16, "f32", torch.bfloat16)]
