@@ -30,6 +30,7 @@ struct FinalizeArgs {
     int64_t tokens;
     int64_t hidden;
     int64_t expandedRows;  // rows of expandedX viewed as 2-D; indices outside [0, expandedRows) are ignored
+    int64_t biasRows;      // rows of bias; an expert id outside [0, biasRows) adds no bias
     int32_t topK;
     int32_t dropPadMode;
 };
@@ -126,9 +127,11 @@ __global__ __launch_bounds__(256) void FinalizeKernel(FinalizeArgs a, int scaleI
             for (int i = 0; i < kVec; ++i) v[i] = Codec::Load(row.v[i]);
             if (a.bias != nullptr) {
                 const int64_t e = a.expertIdx[token * a.topK + k];
-                const P b = static_cast<const P*>(a.bias)[e * packets + pk];
+                if (e >= 0 && e < a.biasRows) {  // expert ids are caller data: never index the bias table with a bad one
+                    const P b = static_cast<const P*>(a.bias)[e * packets + pk];
 #pragma unroll
-                for (int i = 0; i < kVec; ++i) v[i] = Codec::Round(__fadd_rn(v[i], Codec::Load(b.v[i])));
+                    for (int i = 0; i < kVec; ++i) v[i] = Codec::Round(__fadd_rn(v[i], Codec::Load(b.v[i])));
+                }
             }
 #pragma unroll
             for (int i = 0; i < kVec; ++i) {
@@ -291,6 +294,7 @@ extern "C" aclnnStatus aclnnMoeFinalizeRoutingV2GetWorkspaceSize(
     a.tokens = n;
     a.hidden = h;
     a.expandedRows = h > 0 ? Numel(expandedX) / h : 0;
+    a.biasRows = biasOptional != nullptr ? biasOptional->dims[0] : 0;
     a.topK = static_cast<int32_t>(k);
     a.dropPadMode = static_cast<int32_t>(dropPadMode);
     const int vec = dt == ACL_FLOAT ? 4 : 8;

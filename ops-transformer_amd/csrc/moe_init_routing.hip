@@ -471,6 +471,7 @@ struct QuantGatherArgs {
     int32_t expertStart;
     int32_t dtype;                  // ACL_FLOAT, ACL_FLOAT16, ACL_BF16
     int32_t smoothPerExpert;        // 1: smooth row = expert - expertStart; 0: one row for every expert
+    int32_t smoothRows;             // rows of the smooth scale; a copy whose expert falls outside them is not written
     // static quantisation (MoeInitRoutingQuantV2 quantMode 0): both non-null, one float each; no per-row scale then
     const float* staticScale;
     const float* staticOffset;
@@ -533,9 +534,10 @@ __global__ __launch_bounds__(kGatherThreads) void QuantGatherRowsKernel(QuantGat
     for (int j = 0; j < copies; ++j) {
         const int32_t dstOne = a.expandedRowIdx[n * a.topK + j];
         if (perCopy && (dstOne < 0 || dstOne >= a.limit)) continue;  // uniform over the workgroup
-        const float* smooth = a.smooth == nullptr ? nullptr
-                              : perCopy ? a.smooth + static_cast<int64_t>(a.expertIdx[n * a.topK + j] - a.expertStart) * a.cols
-                                        : a.smooth;
+        // expert ids are caller data: an id outside the smooth scale's rows must not index it
+        const int64_t smoothRow = perCopy ? static_cast<int64_t>(a.expertIdx[n * a.topK + j]) - a.expertStart : 0;
+        if (perCopy && (smoothRow < 0 || smoothRow >= a.smoothRows)) continue;
+        const float* smooth = a.smooth == nullptr ? nullptr : a.smooth + smoothRow * a.cols;
         float mx = 0.f;
         for (int64_t c = static_cast<int64_t>(threadIdx.x) * kVec; c < a.cols && !isStatic; c += kGatherThreads * kVec) {
             float v[kVec];
@@ -631,6 +633,7 @@ class InitRoutingExecutor : public aclOpExecutor {
     float* expandedScale = nullptr;
     bool dynamicQuant = false;                // quantMode 1: `scale` is the optional smooth scale [active, cols]
     bool smoothPerExpert = true;              // false: the smooth scale is one row [1, cols] for every expert
+    int64_t smoothRows = 0;                   // rows of the smooth scale
     const float* staticScale = nullptr;       // MoeInitRoutingQuantV2 quantMode 0: scale[1], offset[1] on the device
     const float* staticOffset = nullptr;
     int32_t xDtype = ACL_FLOAT;
@@ -819,7 +822,8 @@ class InitRoutingExecutor : public aclOpExecutor {
                 }
                 QuantGatherArgs q{x, reinterpret_cast<int8_t*>(expandedX), expandedScale, expandedRowIdx, expertIdx,
                                   dynamicQuant ? scale : nullptr, cols, dropPad ? expertNum * capacity : activeRows,
-                                  static_cast<int32_t>(topK), expertStart, xDtype, smoothPerExpert ? 1 : 0, staticScale,
+                                  static_cast<int32_t>(topK), expertStart, xDtype, smoothPerExpert ? 1 : 0,
+                                  static_cast<int32_t>(smoothRows), staticScale,
                                   staticOffset};
                 const bool wide = cols % 4 == 0 && reinterpret_cast<uintptr_t>(expandedX) % 4 == 0 &&
                                   reinterpret_cast<uintptr_t>(x) % 16 == 0;
@@ -983,6 +987,7 @@ aclnnStatus PlanRoutingV2(const aclTensor* x, const aclTensor* expertIdx, const 
         ex->dynamicQuant = true;
         OPAPI_BIND(ex, scaleOptional, &ex->scale);
         ex->smoothPerExpert = smoothPerExpert;
+        ex->smoothRows = scaleOptional != nullptr ? scaleOptional->dims[0] : 0;
         ex->expandedScale = reinterpret_cast<float*>(DataPtr(dynamicQuantScaleOut));
     }
     ex->xDtype = x->dtype;
@@ -1176,6 +1181,7 @@ extern "C" aclnnStatus aclnnMoeInitRoutingV3GetWorkspaceSize(
     OPAPI_BIND(ex, scaleOptional, &ex->scale);
     ex->expandedScale = (dynamicQuant || scaleOptional != nullptr) ? reinterpret_cast<float*>(DataPtr(expandedScaleOut)) : nullptr;
     ex->dynamicQuant = dynamicQuant;
+    ex->smoothRows = (dynamicQuant && scaleOptional != nullptr) ? scaleOptional->dims[0] : 0;
     ex->xDtype = x->dtype;
     ex->cols = cols;
     ex->expertStart = static_cast<int32_t>(expertStart);
