@@ -1,7 +1,7 @@
 """Benchmark of the quantized MoE expert-FFN path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline] [--calibration-copy]
-                    [--fused-combine] [--graph] [--weight-nz]
+                    [--fused-combine] [--graph] [--weight-nz | --weight-row-major]
 
 A step is one pass of the path (routing -> gate/up GEMM + SwiGLU + requant -> down GEMM -> finalize) over one batch of
 synthetic tokens whose inputs and expert weights are already resident in HBM.  Prints ONE JSON line: tokens/s for the
@@ -91,6 +91,8 @@ def main():
                     help="replay the pass from a HIP graph (second phases only) instead of calling the operators eagerly")
     ap.add_argument("--weight-nz", action="store_true",
                     help="give the GEMM operators FRACTAL_NZ weights ([E, N/32, K/16, 16, 32]) instead of transposed views")
+    ap.add_argument("--weight-row-major", action="store_true",
+                    help="give the GEMM operators contiguous row-major [E, K, N] weights (the reference's plain ND layout)")
     ap.add_argument("--fused-combine", action="store_true",
                     help="end the chain with aclnnGroupedMatmulFinalizeRoutingV3 instead of GroupedMatmulV4 + MoeFinalizeRoutingV2")
     args = ap.parse_args()
@@ -113,7 +115,8 @@ def main():
     idx, wgt = pkg.synth.make_routing(cfg, seed=seed)
     xq, xs = pkg.synth.make_activations(cfg, seed=seed)
     w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=seed)
-    ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, fused_combine=args.fused_combine, weight_nz=args.weight_nz)
+    ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, fused_combine=args.fused_combine, weight_nz=args.weight_nz,
+                         weight_row_major=args.weight_row_major)
     d_xq, d_xs = torch.from_numpy(xq).to(dev), torch.from_numpy(xs).to(dev)
     d_idx, d_wgt = torch.from_numpy(idx).to(dev), torch.from_numpy(wgt).to(dev)
 
@@ -193,7 +196,8 @@ def main():
         "config": {"workload": "%s: %d tokens, H=%d, I=%d, E=%d, top-%d, %s routing" % (
             cfg.name, cfg.tokens, cfg.hidden, cfg.inter, cfg.experts, cfg.top_k,
             "Zipf(%.1f)" % cfg.skew if cfg.skew else "uniform random"),
-            "expanded_rows": M, "experts_touched": touched, "weight_layout": "FRACTAL_NZ" if args.weight_nz else "K-contiguous (transposed view)",
+            "expanded_rows": M, "experts_touched": touched, "weight_layout": "FRACTAL_NZ" if args.weight_nz else "row-major [E, K, N]" if args.weight_row_major
+            else "K-contiguous (transposed view)",
             "chain": "V3 routing, SwiGLU GEMM, " + ("fused down GEMM + combine" if args.fused_combine else "down GEMM, finalize"),
             "launch": "HIP graph replay" if args.graph else "eager two-phase calls"},
         "end_to_end": {"tops": work["ops"] / (elapsed / args.steps) / 1e12, "gbps": work["bytes"] / (elapsed / args.steps) / 1e9,

@@ -34,10 +34,11 @@ class MoeFfnW8A8:
     """
 
     def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v3", fused_combine=False,
-                 weight_nz=False):
+                 weight_nz=False, weight_row_major=False):
         assert routing in ("v2", "v3")
         assert not (fused_combine and routing != "v3")
         assert not (fused_combine and weight_nz)
+        assert not (weight_nz and weight_row_major)
         self.routing = routing
         self.fused_combine = fused_combine
         # weight_nz: hand the operators the reference's FRACTAL_NZ weights ([E, N/32, K/16, 16, 32]) instead of the
@@ -47,6 +48,10 @@ class MoeFfnW8A8:
         assert w13.dtype == torch.int8 and w2.dtype == torch.int8
         self.w13_view = w13.transpose(1, 2)  # [E, H, 2I]
         self.w2_view = w2.transpose(1, 2)    # [E, I, H]
+        if weight_row_major:
+            # the reference's plain ND layout: contiguous [E, K, N] copies, made here, once
+            self.w13_view = self.w13_view.contiguous()
+            self.w2_view = self.w2_view.contiguous()
         self.w13_scale = w13_scale
         self.w2_scale = w2_scale
         self.num_experts = w13.shape[0]
