@@ -588,9 +588,10 @@ __device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leavi
 //
 // kNMajor: the weights are row-major [K, N] per expert (N contiguous), the reference's plain ND layout of the grouped
 // matmul.  A stage's weight part is then 128 k-rows of the tile's 256 channel bytes (one 256-byte run per k-row, two of
-// 128 bytes for the gate and up halves of a SwiGLU tile); it lies in LDS as [k][256] with the 16-byte chunks of row k
-// XOR-ed by k & 15, and the operands come out through the same transposing load as for the blocked layout (8
-// consecutive k-rows then sit in 8 different bank groups).
+// 128 bytes for the gate and up halves of a SwiGLU tile); it lies in LDS as [k][256] with the 16-byte chunk index of row
+// k XOR-ed by 2 * (k & 7), and the operands come out through the same transposing load as for the blocked layout: the
+// 32 lanes the LDS serves together read one pair of neighbouring chunks from each of 8 consecutive k-rows, and the
+// swizzle puts those 8 pairs into 8 different bank groups (a row of 256 bytes spans all 64 banks once).
 template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor = false>
 __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     KernelArgs a, const int32_t* __restrict__ sched) {
@@ -659,7 +660,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                 // Chunks past the last channel are never stored: such lanes re-read the last real chunk.
                 const int jw = j - Cfg::kInstrA;
                 const int k = 4 * jw + lane / 16;
-                const int c = (lane % 16) ^ (k & 15);
+                const int c = (lane % 16) ^ ((k & 7) << 1);
                 int32_t col;
                 if (kSwiglu) {
                     col = c < 8 ? min(iss.colBase + 16 * c, a.halfN - 16) : min(a.halfN + iss.colBase + 16 * (c - 8), a.N - 16);
@@ -758,8 +759,9 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
 #pragma unroll
                     for (int ni = 0; ni < 2; ++ni) {
                         const int c = (bRow0 + ni * bRowStep + 16 * ((lane >> 4) & 1)) >> 4;  // logical 16-byte chunk of the row
-                        const uint32_t lo = bBase + k * 256 + ((c ^ (k & 15)) << 4);
-                        const uint32_t hi = bBase + (k + 8) * 256 + ((c ^ ((k + 8) & 15)) << 4);
+                        // k and k + 8 share their low three bits, hence their swizzle
+                        const uint32_t lo = bBase + k * 256 + ((c ^ ((k & 7) << 1)) << 4);
+                        const uint32_t hi = lo + 8 * 256;
                         const v2i vlo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(lo));
                         const v2i vhi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(hi));
                         bf[buf][ni] = v4i{vlo[0], vlo[1], vhi[0], vhi[1]};
