@@ -191,6 +191,7 @@ struct KernelArgs {
     int64_t wStrideN;      // bytes between consecutive output channels
     int64_t wStrideK;      // bytes between consecutive k
     int32_t wNz;           // weights in 32-channel x 16-k blocks ([N/32][K/16][16][32] per expert), see Problem::wNz
+    int32_t rotateK;       // ring kernel: every workgroup starts its k walk at its own offset
     int32_t M, K, N;
     int32_t groups;
     int32_t tilesN;
@@ -625,6 +626,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     TileInfo cur = decode(local);
     if (!cur.valid) return;
     const int kSteps = a.K / kStep;
+    const int kRotate = a.rotateK ? static_cast<int>((blockIdx.x * 7u + blockIdx.x / kXcds) % static_cast<unsigned>(kSteps)) : 0;
 
     // ---- issue side: runs kStages - 1 steps ahead of the compute side, across tile boundaries ----
     const uint32_t ldsBase = LdsAddress(lds);
@@ -683,7 +685,14 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     };
     auto issueStage = [&](int ring) {
         const uint32_t dst = ldsBase + ring * kStageBytes;
-        const int kOff = issStep * kStep;
+        // With a.rotateK the k-steps of a tile are walked from a start that differs between workgroups (integer
+        // accumulation does not care about the order).  When rows lie a power-of-two stride apart (K = 4096 with
+        // K-contiguous weights), the low address bits of every row of every expert depend on the k offset alone:
+        // workgroups that all sit at the same k-step all queue on the same memory channels.  Only for small tiles, where
+        // every weight byte is used once: on the large-tile shapes neighbouring workgroups share operands through L2,
+        // and walking k in step is what makes those hits.
+        const int kIdx = issStep + kRotate;
+        const int kOff = (kIdx >= kSteps ? kIdx - kSteps : kIdx) * kStep;
         // blocked layout: one k is 32 bytes further; row-major: N bytes
         const int kOffW = kNz ? kOff * 32 : (kNMajor ? kOff * a.N : kOff);
 #pragma unroll
@@ -1129,6 +1138,7 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.wStrideN = p.wKMajor ? p.K : 1;
     ka.wStrideK = p.wNz ? 32 : (p.wKMajor ? 1 : p.N);
     ka.wNz = p.wNz ? 1 : 0;
+    ka.rotateK = plan.tileM <= 64 ? 1 : 0;
     ka.M = static_cast<int32_t>(p.M);
     ka.K = static_cast<int32_t>(p.K);
     ka.N = static_cast<int32_t>(p.N);
