@@ -165,3 +165,44 @@ def test_finalize_random(aclnn, oracle, dev, seed):
     g = got.cpu()
     g = g.numpy() if name == "f32" else g.view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(g, want), (T, K, E, H, mode, name)
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_routing_quant_v2_random(aclnn, oracle, dev, seed):
+    rng = np.random.default_rng(5000 + seed)
+    T, K = int(rng.integers(1, 300)), int(rng.integers(1, 9))
+    E = int(rng.choice([1, 2, 7, 64, 256, 512, 513, 2048]))
+    H = int(rng.integers(1, 150)) if seed % 2 else int(rng.integers(1, 40)) * 4
+    name = ["f32", "f16", "bf16"][seed % 3]
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[name]
+    code = {"f32": oracle.DT_F32, "f16": oracle.DT_F16, "bf16": oracle.DT_BF16}[name]
+    quant = seed % 2
+    xt = torch.from_numpy((rng.standard_normal((T, H)) * (2 if quant else 60)).astype(np.float32)).to(tdt)
+    bits = xt.numpy() if name == "f32" else xt.view(torch.int16).numpy().view(np.uint16)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    if quant == 0:
+        scale, offset = np.float32(rng.uniform(0.2, 2.0)), np.float32(rng.uniform(-5, 5))
+        s_t = torch.tensor([scale], dtype=torch.float32, device=dev)
+        o_t = torch.tensor([offset], dtype=torch.float32, device=dev)
+        s_o, o_o = scale, offset
+    else:
+        rows = [None, 1, E][seed % 3]
+        smooth = None if rows is None else (rng.random((rows, H)) + 0.5).astype(np.float32)
+        s_t, o_t = (None if smooth is None else torch.from_numpy(smooth).to(dev)), None
+        s_o, o_o = smooth, None
+    if seed % 4 >= 2:
+        C = int(rng.integers(1, T + 1))
+        kw = dict(expert_num=E, expert_capacity=C, drop_pad_mode=1, expert_tokens_before_capacity_flag=bool(seed % 8 >= 6))
+        okw = dict(expert_num=E, expert_capacity=C, drop_pad_mode=1, before_capacity_flag=kw["expert_tokens_before_capacity_flag"])
+    else:
+        active = int(rng.integers(0, T * K + 5)) if seed % 3 == 0 else 0
+        flag = int(rng.integers(0, 3))
+        kw = dict(expert_num=E, active_num=active, expert_tokens_count_or_cumsum_flag=flag)
+        okw = dict(expert_num=E, active_num=active, count_flag=flag)
+    got = aclnn.moe_init_routing_quant_v2(xt.to(dev), torch.from_numpy(idx).to(dev), quant, s_t, o_t, **kw)
+    torch.cuda.synchronize()
+    want = oracle.moe_init_routing_quant_v2(bits, idx, quant, s_o, o_o, dtype=code, **okw)
+    for g, w, label in zip(got, want, ("expandedX", "expandedRowIdx", "countOrCumsum", "beforeCapacity", "dynamicQuantScale")):
+        assert (g is None) == (w is None), label
+        if g is not None:
+            assert np.array_equal(_np(g), w), (label, quant, kw, T, K, E, H, name)
