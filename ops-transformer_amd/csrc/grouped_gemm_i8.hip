@@ -191,7 +191,6 @@ struct KernelArgs {
     int64_t wStrideN;      // bytes between consecutive output channels
     int64_t wStrideK;      // bytes between consecutive k
     int32_t wNz;           // weights in 32-channel x 16-k blocks ([N/32][K/16][16][32] per expert), see Problem::wNz
-    int32_t rotateK;       // ring kernel: every workgroup starts its k walk at its own offset
     int32_t M, K, N;
     int32_t groups;
     int32_t tilesN;
@@ -567,10 +566,17 @@ __device__ __forceinline__ uint32_t LdsAddress(const char* p) {
 // 16 bytes per lane from (uniform base + 32-bit lane offset) straight into LDS at ldsAddr + lane * 16 (ldsAddr is the
 // 32-bit LDS address, see LdsAddress).  The compiler does not see this as a memory instruction: completion is awaited
 // with WaitVmcnt below.
+// kStreaming marks the load non-temporal: the bytes are used once (weights), so they should not push the operands
+// that are re-read from L2 (activation rows) out of the caches.
+template <bool kStreaming>
 __device__ __forceinline__ void DmaToLdsAddr16(const char* base, uint32_t laneOffset, uint32_t ldsAddr) {
     const uint32_t m0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(ldsAddr)));
     const char* const sbase = UniformPtr(base);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(laneOffset), "s"(sbase) : "memory");
+    if (kStreaming) {
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0), "v"(laneOffset), "s"(sbase) : "memory");
+    } else {
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(laneOffset), "s"(sbase) : "memory");
+    }
 }
 
 template <int kCount>
@@ -620,13 +626,15 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
     const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
     const int64_t slots = gridDim.x / kXcds;
-    auto decode = [&](int64_t local) { return DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, local); };
+    auto decode = [&](int64_t local) __attribute__((always_inline)) { return DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, local); };
 
     int64_t local = blockIdx.x / kXcds;
     TileInfo cur = decode(local);
     if (!cur.valid) return;
     const int kSteps = a.K / kStep;
-    const int kRotate = a.rotateK ? static_cast<int>((blockIdx.x * 7u + blockIdx.x / kXcds) % static_cast<unsigned>(kSteps)) : 0;
+    // Small tiles are the decode shapes: a handful of rows per expert, every weight byte used once, pure streaming.
+    constexpr bool kSmallTile = kTileM <= 64;
+    const int kRotate = kSmallTile ? static_cast<int>((blockIdx.x * 7u + blockIdx.x / kXcds) % static_cast<unsigned>(kSteps)) : 0;
 
     // ---- issue side: runs kStages - 1 steps ahead of the compute side, across tile boundaries ----
     const uint32_t ldsBase = LdsAddress(lds);
@@ -639,7 +647,9 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     // Every wave issues exactly kMaxPerWave DMA instructions per stage: slots past the last instruction repeat it (same
     // bytes to the same place), which keeps the issue code free of branches and the vmcnt arithmetic uniform.
 
-    auto setupIssue = [&]() {
+    // The lambdas below are forced inline: left to the inliner's size heuristics, one of them staying a real call puts
+    // the whole issue state (captured by reference) into scratch memory and the kernel runs three times slower.
+    auto setupIssue = [&]() __attribute__((always_inline)) {
         issX = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(iss.rowBase) * a.K;
         issW = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(iss.group) * a.wGroupStride;
         // lane -> (row inside the instruction, LDS chunk slot); the global chunk it fetches is the one LdsOffset puts there
@@ -683,9 +693,9 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             }
         }
     };
-    auto issueStage = [&](int ring) {
+    auto issueStage = [&](int ring) __attribute__((always_inline)) {
         const uint32_t dst = ldsBase + ring * kStageBytes;
-        // With a.rotateK the k-steps of a tile are walked from a start that differs between workgroups (integer
+        // On small tiles the k-steps of a tile are walked from a start that differs between workgroups (integer
         // accumulation does not care about the order).  When rows lie a power-of-two stride apart (K = 4096 with
         // K-contiguous weights), the low address bits of every row of every expert depend on the k offset alone:
         // workgroups that all sit at the same k-step all queue on the same memory channels.  Only for small tiles, where
@@ -698,7 +708,15 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
             const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
-            DmaToLdsAddr16(j < Cfg::kInstrA ? issX + kOff : issW + kOffW, laneOff[q], dst + j * 1024);
+            // wave-uniform branch: activation rows always stay cacheable (the n-tiles of a group re-read them from L2);
+            // on small tiles (every weight byte is used exactly once) the weights stream past the caches.  On large
+            // tiles the m-tiles of a group share their weight columns through L2 and must not.
+            if constexpr (kSmallTile) {
+                if (j < Cfg::kInstrA) DmaToLdsAddr16<false>(issX + kOff, laneOff[q], dst + j * 1024);
+                else DmaToLdsAddr16<true>(issW + kOffW, laneOff[q], dst + j * 1024);
+            } else {
+                DmaToLdsAddr16<false>(j < Cfg::kInstrA ? issX + kOff : issW + kOffW, laneOff[q], dst + j * 1024);
+            }
         }
         if (++issStep == kSteps) {
             // move to this workgroup's next tile; past the last one the same tile is fetched again into ring slots
@@ -749,14 +767,14 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         // One k-step of a wave with kMy MFMA tiles: straight-line code, the operands of k-slice ks + 1 are read
         // from LDS before the MFMAs of k-slice ks are issued, and the refill of the stage freed by the barrier goes out
         // behind the first block of MFMAs (its scalar address work then runs in the shadow of the matrix pipe).
-        auto computeStep = [&](auto myTag) {
+        auto computeStep = [&](auto myTag) __attribute__((always_inline)) {
             constexpr int kMy = decltype(myTag)::value;
             const char* const A = lds + ring * kStageBytes;
             const char* const B = A + kTileM * kStep;
             constexpr int kSlices = kStep / 32;
             v4i bf[2][2];
             v4i af[2][kMy > 0 ? kMy : 1];
-            auto loadSlice = [&](int ks, int buf) {
+            auto loadSlice = [&](int ks, int buf) __attribute__((always_inline)) {
                 if (kMy == 0) return;
                 const int chunk = 2 * ks + lhi;
                 if constexpr (kNMajor) {
@@ -811,7 +829,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             }
         };
 
-        auto runTile = [&](auto myTag) {
+        auto runTile = [&](auto myTag) __attribute__((always_inline)) {
 #pragma unroll 1
             for (int step = 0; step < kSteps; ++step) {
                 // the oldest stage in flight has landed once at most (kStages - 2) stages' worth of this wave's DMAs remain
@@ -1138,7 +1156,6 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.wStrideN = p.wKMajor ? p.K : 1;
     ka.wStrideK = p.wNz ? 32 : (p.wKMajor ? 1 : p.N);
     ka.wNz = p.wNz ? 1 : 0;
-    ka.rotateK = plan.tileM <= 64 ? 1 : 0;
     ka.M = static_cast<int32_t>(p.M);
     ka.K = static_cast<int32_t>(p.K);
     ka.N = static_cast<int32_t>(p.N);
