@@ -333,7 +333,7 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                         const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
                         const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
                         uint16_t* const rowPtr = outTile + static_cast<int64_t>(32 * mi + 8 * q + i) * a.N;
-                        if (full || rTop + 8 * q + 4 * lhi + i < rows) *reinterpret_cast<uint32_t*>(rowPtr + laneOff) = word;
+                        if (full || rTop + 8 * q + 4 * lhi + i < rows) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t*>(rowPtr + laneOff));
                     }
                 }
             }
@@ -433,7 +433,7 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                         const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xsv[i]), scB);
                         float sv = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
                         const bool ok = full || rTop + 8 * q + 4 * lhi + i < rows;
-                        if (ok) sTile[static_cast<int64_t>(8 * q + i) * a.halfN + laneOff] = sv;
+                        if (ok) __builtin_nontemporal_store(sv, &sTile[static_cast<int64_t>(8 * q + i) * a.halfN + laneOff]);
                         m[v] = ok ? fabsf(sv) : 0.0f;
                     }
                 }
@@ -990,13 +990,15 @@ __global__ __launch_bounds__(256) void RequantKernel(RequantArgs a) {
     const bool zeroRow = mx == 0.0f;  // reference: 0 * inf; defined here as zeros
     if ((a.halfN & 3) == 0) {
         for (int j = threadIdx.x * 4; j < a.halfN; j += 256 * 4) {
-            const float4 v = *reinterpret_cast<const float4*>(src + j);
+            // S is read exactly once: a non-temporal load keeps it from displacing anything in the caches
+            typedef float Float4 __attribute__((ext_vector_type(4)));
+            const Float4 v = __builtin_nontemporal_load(reinterpret_cast<const Float4*>(src + j));
             char4 q;
             q.x = zeroRow ? 0 : QuantOne(v.x, inv);
             q.y = zeroRow ? 0 : QuantOne(v.y, inv);
             q.z = zeroRow ? 0 : QuantOne(v.z, inv);
             q.w = zeroRow ? 0 : QuantOne(v.w, inv);
-            *reinterpret_cast<char4*>(dst + j) = q;
+            *reinterpret_cast<char4*>(dst + j) = q;  // read again soon, by the down projection: stays cacheable
         }
     } else {
         for (int j = threadIdx.x; j < a.halfN; j += 256) dst[j] = zeroRow ? 0 : QuantOne(src[j], inv);
