@@ -115,17 +115,21 @@ def test_graph_replays_match_eager(pkg, dev):
         assert torch.equal(out.view(torch.int16), want.view(torch.int16)), seed
 
 
-def test_nz_weight_chain_equals_nd_chain(pkg, dev):
-    """The chain fed FRACTAL_NZ weights equals the chain fed the transposed views, bit for bit."""
-    cfg = pkg.synth.config(0)
+@pytest.mark.parametrize("config", [0, 3])
+def test_nz_weight_chain_equals_nd_chain(pkg, dev, config):
+    """The chain fed FRACTAL_NZ weights, and the chain fed contiguous row-major [E, K, N] weights, equal the chain fed
+    the transposed views of K-contiguous storage, bit for bit (c0, and the decode shape c3 with its 32-row tiles)."""
+    cfg = pkg.synth.config(config)
     idx, wgt = pkg.synth.make_routing(cfg, seed=0)
     xq, xs = pkg.synth.make_activations(cfg, seed=0)
     w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=0)
     t = lambda a: torch.from_numpy(a).to(dev)
     a = pkg.MoeFfnW8A8(w13, w13s, w2, w2s).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
     b = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, weight_nz=True).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
+    c = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, weight_row_major=True).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
     torch.cuda.synchronize()
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert torch.equal(a.view(torch.int16), c.view(torch.int16))
 
 
 def test_two_host_threads_on_their_own_streams(pkg, dev):
