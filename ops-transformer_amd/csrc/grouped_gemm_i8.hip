@@ -308,8 +308,9 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
         const bool pairStores = kEpi == Epilogue::kDequant && a.outDtype != 0 && (a.N & 1) == 0 &&
                                 t.colBase + 64 * waveN + 64 <= a.N;  // wave-uniform
         const bool oddLane = (l32 & 1) != 0;
-        if (kEpi == Epilogue::kDequant && a.outDtype == 27 && pairStores) {
-            // The common case (bf16 output, whole column pairs) without per-element dtype dispatch: row scales come
+        if (kEpi == Epilogue::kDequant && (a.outDtype == 27 || a.outDtype == 1) && pairStores) {
+            const bool toBf16 = a.outDtype == 27;  // wave-uniform: bf16, else fp16
+            // The common case (16-bit output, whole column pairs) without per-element dtype dispatch: row scales come
             // from LDS four at a time, every lane stores one 32-bit word per accumulator pair through a
             // (uniform row pointer + 32-bit lane offset) address.
             uint16_t* const outTile = static_cast<uint16_t*>(a.out) + static_cast<int64_t>(rowBase + waveRow0) * a.N;
@@ -329,7 +330,9 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                         const int v = 4 * q + i;
                         const Float2 f = {__fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), sc0), rsv[i]),
                                           __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), sc1), rsv[i])};
-                        const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));
+                        const uint32_t pk = toBf16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2))
+                                                   : (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[0]))) |
+                                                      (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[1]))) << 16));
                         const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
                         const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
                         uint16_t* const rowPtr = outTile + static_cast<int64_t>(32 * mi + 8 * q + i) * a.N;
