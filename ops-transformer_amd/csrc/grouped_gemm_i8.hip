@@ -644,6 +644,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     TileInfo iss = cur;
     int64_t issLocal = local;
     int issStep = 0;
+    bool issDrained = false;  // no further tile: the remaining issue slots re-read one hot kilobyte (see below)
     const char* issX = nullptr;
     const char* issW = nullptr;
     uint32_t laneOff[Cfg::kMaxPerWave];
@@ -705,7 +706,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         // every weight byte is used once: on the large-tile shapes neighbouring workgroups share operands through L2,
         // and walking k in step is what makes those hits.
         const int kIdx = issStep + kRotate;
-        const int kOff = (kIdx >= kSteps ? kIdx - kSteps : kIdx) * kStep;
+        const int kOff = issDrained ? 0 : (kIdx >= kSteps ? kIdx - kSteps : kIdx) * kStep;
         // blocked layout: one k is 32 bytes further; row-major: N bytes
         const int kOffW = kNz ? kOff * 32 : (kNMajor ? kOff * a.N : kOff);
 #pragma unroll
@@ -722,15 +723,22 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             }
         }
         if (++issStep == kSteps) {
-            // move to this workgroup's next tile; past the last one the same tile is fetched again into ring slots
-            // nobody reads, which keeps the number of outstanding DMAs per stage constant
+            // move to this workgroup's next tile.  Past the last one the issue slots still go out (that keeps the number
+            // of outstanding DMAs per stage, hence the vmcnt arithmetic, constant) into ring slots nobody reads -- but
+            // every one of them then re-reads the same first kilobyte of the last tile's weights, which stays in L2,
+            // instead of pulling (stages - 1) more stages of weights from HBM per workgroup.
             issStep = 0;
             const TileInfo next = decode(issLocal + slots);
             if (next.valid) {
                 iss = next;
                 issLocal += slots;
+                setupIssue();
+            } else if (!issDrained) {
+                issDrained = true;
+                issX = issW;  // any mapped, 16-byte aligned kilobyte will do
+#pragma unroll
+                for (int q = 0; q < Cfg::kMaxPerWave; ++q) laneOff[q] = static_cast<uint32_t>(lane) * kChunk;
             }
-            setupIssue();
         }
     };
 
