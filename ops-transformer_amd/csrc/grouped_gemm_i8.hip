@@ -571,6 +571,9 @@ __device__ __forceinline__ uint32_t LdsAddress(const char* p) {
 // with WaitVmcnt below.
 // kStreaming marks the load non-temporal: the bytes are used once (weights), so they should not push the operands
 // that are re-read from L2 (activation rows) out of the caches.
+// The instruction takes its LDS base from m0, which the statement sets itself.  m0 is a reserved register that cannot
+// be named as a clobber; nothing else in these kernels uses it (no LDS-direct or register-indexed code is generated
+// for them), and the compiler sets m0 afresh before any use of its own.
 template <bool kStreaming>
 __device__ __forceinline__ void DmaToLdsAddr16(const char* base, uint32_t laneOffset, uint32_t ldsAddr) {
     const uint32_t m0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(ldsAddr)));
