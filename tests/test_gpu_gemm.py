@@ -319,3 +319,38 @@ def test_grouped_matmul_nz_weight(aclnn, oracle, dev, M, K, N, E, mode, how):
     assert np.array_equal(acc.cpu().numpy()[:rows], oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)[:rows])
     ref = oracle.grouped_matmul_dequant(x, wt, scale, pt, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
     assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16)[:rows], ref[:rows])
+
+
+# ------------------------------------------------------------------------------------------------ every instantiation
+@pytest.mark.parametrize("layout", ["kmajor", "nz", "nd"])
+@pytest.mark.parametrize("tile_m", [32, 64, 96, 128, 160, 192, 256])
+def test_every_tile_height_and_layout(aclnn, oracle, dev, monkeypatch, tile_m, layout):
+    """The fast kernel is compiled once per (tile height, weight layout, epilogue).  The planner picks the height from the
+    group sizes, so the hand-picked shapes reach only some of the 63; here the height is forced and one ragged problem
+    (groups of 0 to ~400 rows, a partial n-tile) runs through all three epilogues of each one: int32 and bf16 bit-exact,
+    SwiGLU-quant to +-1 LSB."""
+    monkeypatch.setenv("OPAPI_GEMM_TILE_M", str(tile_m))
+    rng = np.random.default_rng(77)
+    M, K, N, E = 900, 384, 320, 6
+    x, wt, cumsum = _problem(rng, M, K, N, E, "ragged")
+    cumsum[1] = cumsum[0]                                        # one empty group
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    if layout == "nz":
+        w_nz = t(_to_nz(np.ascontiguousarray(wt.transpose(0, 2, 1))))
+        wkw, wv, wsw = dict(weight_nz=(w_nz, "nz5d")), None, dict(weight_nz=(w_nz, "nz5d"))
+    else:
+        wkw, wv, wsw = {}, [_weight_views(wt, dev, layout)], {}
+    acc = aclnn.grouped_matmul_v4([t(x)], wv, group_list=t(cumsum), split_item=3, group_type=0, **wkw)[0]
+    y = aclnn.grouped_matmul_v4([t(x)], wv, scale=[t(scale)], per_token_scale=[t(pt)], group_list=t(cumsum), split_item=3,
+                                group_type=0, output_dtype=torch.bfloat16, **wkw)[0]
+    q, qs = aclnn.grouped_matmul_swiglu_quant(t(x), wv[0] if wv else None, t(cumsum), t(scale), t(pt), **wsw)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True))
+    ref = oracle.grouped_matmul_dequant(x, wt, scale, pt, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+    q_ref, qs_ref = oracle.grouped_matmul_swiglu_quant(x, wt, scale, pt, cumsum, w_trans=True)
+    diff = np.abs(q.cpu().numpy().astype(np.int32) - q_ref.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+    np.testing.assert_allclose(qs.cpu().numpy(), qs_ref, rtol=1e-5)
