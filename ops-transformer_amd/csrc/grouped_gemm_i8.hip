@@ -983,36 +983,51 @@ __device__ __forceinline__ int8_t QuantOne(float s, float inv) {
 }
 
 // One workgroup per row; rows at or beyond the last group boundary are left untouched.
+// Every thread requests its first two packets of S before the row maximum is known, and every wave folds the partial
+// maxima for itself (a handful of L2 hits): the row's two dependent memory round trips overlap and there is no barrier.
 __global__ __launch_bounds__(256) void RequantKernel(RequantArgs a) {
     const int64_t row = blockIdx.x;
     if (row >= a.sched[0]) return;
-    __shared__ float rowMaxShared;
-    if (threadIdx.x < 64) {  // the first wave folds the per-n-tile partial maxima
-        float m = 0.0f;
-        for (int t = threadIdx.x; t < a.tilesN; t += 64) m = fmaxf(m, a.rowMax[static_cast<int64_t>(t) * a.M + row]);
+    typedef float Float4 __attribute__((ext_vector_type(4)));
+    const float* src = a.s + row * a.halfN;
+    int8_t* dst = a.y + row * a.halfN;
+    const bool packets = (a.halfN & 3) == 0;
+    constexpr int kAhead = 2;
+    Float4 ahead[kAhead];
+    if (packets) {
 #pragma unroll
-        for (int d = 1; d < 64; d <<= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
-        if (threadIdx.x == 0) rowMaxShared = m;
+        for (int i = 0; i < kAhead; ++i) {
+            const int j = (static_cast<int>(threadIdx.x) + 256 * i) * 4;
+            // S is read exactly once: a non-temporal load keeps it from displacing anything in the caches
+            ahead[i] = j < a.halfN ? __builtin_nontemporal_load(reinterpret_cast<const Float4*>(src + j)) : Float4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
     }
-    __syncthreads();
-    const float mx = rowMaxShared;
+    float mx = 0.0f;
+    for (int t = threadIdx.x & 63; t < a.tilesN; t += 64) mx = fmaxf(mx, a.rowMax[static_cast<int64_t>(t) * a.M + row]);
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
     const float ys = __fdiv_rn(mx, 127.0f);
     const float inv = __fdiv_rn(1.0f, ys);
     if (threadIdx.x == 0) a.yScale[row] = ys;
-    const float* src = a.s + row * a.halfN;
-    int8_t* dst = a.y + row * a.halfN;
     const bool zeroRow = mx == 0.0f;  // reference: 0 * inf; defined here as zeros
-    if ((a.halfN & 3) == 0) {
-        for (int j = threadIdx.x * 4; j < a.halfN; j += 256 * 4) {
-            // S is read exactly once: a non-temporal load keeps it from displacing anything in the caches
-            typedef float Float4 __attribute__((ext_vector_type(4)));
-            const Float4 v = __builtin_nontemporal_load(reinterpret_cast<const Float4*>(src + j));
+    if (packets) {
+        auto quantPacket = [&](const Float4 v, int j) __attribute__((always_inline)) {
             char4 q;
             q.x = zeroRow ? 0 : QuantOne(v.x, inv);
             q.y = zeroRow ? 0 : QuantOne(v.y, inv);
             q.z = zeroRow ? 0 : QuantOne(v.z, inv);
             q.w = zeroRow ? 0 : QuantOne(v.w, inv);
             *reinterpret_cast<char4*>(dst + j) = q;  // read again soon, by the down projection: stays cacheable
+        };
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+            const int j = (static_cast<int>(threadIdx.x) + 256 * i) * 4;
+            if (j < a.halfN) quantPacket(ahead[i], j);
+        }
+        // rows longer than 2048 columns: one packet per trip (batching four loads per trip measured 5 % slower on
+        // 14336-column rows)
+        for (int j = (static_cast<int>(threadIdx.x) + 256 * kAhead) * 4; j < a.halfN; j += 256 * 4) {
+            quantPacket(__builtin_nontemporal_load(reinterpret_cast<const Float4*>(src + j)), j);
         }
     } else {
         for (int j = threadIdx.x; j < a.halfN; j += 256) dst[j] = zeroRow ? 0 : QuantOne(src[j], inv);
