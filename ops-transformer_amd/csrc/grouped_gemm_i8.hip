@@ -75,18 +75,21 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
         return a.groupListIsInt64 ? static_cast<const int64_t*>(a.groupList)[i]
                                   : static_cast<int64_t>(static_cast<const int32_t*>(a.groupList)[i]);
     };
+    // inclusive prefix sum over the 1024 threads: shuffles inside each wave, then the sixteen wave totals through LDS
+    __shared__ int32_t waveTotal[16];
     auto inclusiveScan = [&](int32_t v) -> int32_t {
-        scan[t] = v;
-        __syncthreads();
-        for (int d = 1; d < 1024; d <<= 1) {
-            const int32_t add = t >= d ? scan[t - d] : 0;
-            __syncthreads();
-            scan[t] += add;
-            __syncthreads();
+        const int lane = t & 63, wave = t >> 6;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int32_t below = __shfl_up(v, d, 64);
+            if (lane >= d) v += below;
         }
-        const int32_t r = scan[t];
+        __syncthreads();  // the totals of an earlier call have been read
+        if (lane == 63) waveTotal[wave] = v;
         __syncthreads();
-        return r;
+        int32_t base = 0;
+        for (int i = 0; i < wave; ++i) base += waveTotal[i];
+        return v + base;
     };
     // group boundaries, clamped into [0, M] and made monotonic so that a malformed list cannot push rows out of range
     int64_t begin = 0, end = 0;
@@ -167,7 +170,7 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
             a.sched[1] = tileInc < a.maxMTiles ? tileInc : a.maxMTiles;
         }
     }
-    // group of every m-tile: scan[] still holds the inclusive m-tile prefix (zero-tile groups repeat their
+    // group of every m-tile: scan[] takes the inclusive m-tile prefix (zero-tile groups repeat their
     // predecessor's value); m-tile m belongs to the first group whose inclusive prefix exceeds m
     scan[t] = t < a.groups ? tileInc : 0x7fffffff;
     __syncthreads();
