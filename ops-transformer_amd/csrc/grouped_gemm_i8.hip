@@ -28,6 +28,7 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <type_traits>
 
@@ -1052,8 +1053,8 @@ template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor
 hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
     using Cfg = StreamCfg<kSub0, kSub1, kStep>;
     auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi, kNz, kNMajor>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes);
+    static std::atomic<uint64_t> optedIn{0};
+    const hipError_t attr = opapi::EnsureDynamicLds(reinterpret_cast<const void*>(kernel), Cfg::kLdsBytes, optedIn);
     if (attr != hipSuccess) return attr;
     // persistent grid: one workgroup per CU (the LDS ring fills the CU), a multiple of the XCD count
     int64_t grid = DeviceCuCount();

@@ -206,9 +206,9 @@ class GatingExecutor : public aclOpExecutor {
         auto kernel = GatingTopKKernel<Codec, kWaves>;
         const size_t lds = LdsBytes(args.cols, args.k, kWaves);
         if (lds > 48 * 1024) {
-            static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                               static_cast<int>(LdsBytes(kMaxCols, kMaxK, kWaves)));
+            static std::atomic<uint64_t> optedIn{0};
+            const hipError_t attr = opapi::EnsureDynamicLds(reinterpret_cast<const void*>(kernel),
+                                                            static_cast<int>(LdsBytes(kMaxCols, kMaxK, kWaves)), optedIn);
             if (attr != hipSuccess) return attr;
         }
         hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(args.rows)), dim3(kWave * kWaves), lds, stream, args);

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -159,6 +160,18 @@ class KernelTimer {
     hipStream_t stream_;
     hipEvent_t start_ = nullptr;
 };
+
+// Raises a kernel's dynamic-LDS limit to `bytes` on the current device.  The opt-in belongs to the kernel as loaded on
+// one device, so it is made once per device of the process; `done` is the caller's per-kernel bit set (one bit per device).
+inline hipError_t EnsureDynamicLds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
+    const uint64_t devBit = 1ull << (dev & 63);
+    if ((done.load(std::memory_order_acquire) & devBit) != 0) return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.fetch_or(devBit, std::memory_order_release);
+    return e;
+}
 
 }  // namespace opapi
 
