@@ -1,19 +1,30 @@
 """Benchmark of the quantized MoE expert-FFN path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline] [--calibration-copy]
-                    [--fused-combine] [--graph] [--weight-nz | --weight-row-major]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline] [--no-other-configs]
+                    [--calibration-copy] [--fused-combine] [--graph] [--routing v2|v3]
+                    [--weight-nz | --weight-row-major]
 
 A step is one pass of the path (routing -> gate/up GEMM + SwiGLU + requant -> down GEMM -> finalize) over one batch of
 synthetic tokens whose inputs and expert weights are already resident in HBM.  Prints ONE JSON line: tokens/s for the
 whole pass, the roofline of the dominant kernel (the gate/up grouped GEMM) from HIP-event durations recorded inside the
 library during the timed steps, and the CPU oracle timed on a bounded sample of the same workload.
 
+The headline (`value`, `roofline`) is the configuration named by --config (default c1, the DeepSeek-V3 prefill shape
+the target is quoted on), run eagerly.  The same line carries, under `other_configs`, a shorter measurement of the other
+halves of the metric: the decode shape c3 (eager and as a HIP-graph replay: HBM-bound), the Mixtral prefill shape c2
+(the MFMA-bound one), the skewed shape c4, and c1 again with aclnnMoeInitRoutingV2 in place of V3 at the head of the
+chain -- each with its ms per pass, per-kernel durations and the gate/up kernel's roofline from the same in-library timer.
+
 --calibration-copy appends, after the timed region, a few launches of the library's plain 1 GiB copy kernel: under
 `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` its counter readings give the factor that converts the counters to
-bytes.  roofline.traffic is read from the text summary of those counter runs under profiles/ (null when there is none
-for the workload): a counter run is a separate profiler pass and cannot happen inside this process.
+bytes.  roofline.traffic is a RECORDED figure: a counter run is a separate profiler pass and cannot happen inside this
+process, so the value is read from the text summary of those counter runs under profiles/, which names the hash of the
+kernel sources it was taken on; it is null when there is no summary for the workload or when the kernel sources have
+changed since (roofline.traffic_source says which).
 """
 import argparse
+import gc
+import hashlib
 import json
 import os
 import sys
@@ -25,8 +36,18 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gmm_swiglu_{config}_hbm_traffic.txt")
+KERNEL_SOURCES = ["grouped_gemm_i8.hip", "grouped_gemm_i8.h", "opapi_common.h"]
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA (5.0 POP/s)
+
+
+def kernel_source_hash():
+    """sha256 (first 16 hex digits) over the source files of the grouped GEMM kernels, in a fixed order."""
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "ops-transformer_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def _cpu_baseline(pkg, oracle, cfg, idx, wgt, xq, xs, ffn, sample_experts=4):
@@ -69,14 +90,161 @@ def _cpu_baseline(pkg, oracle, cfg, idx, wgt, xq, xs, ffn, sample_experts=4):
 
 
 def _recorded_traffic(config_name):
-    """HBM bytes per launch of the gate/up GEMM from the committed counter summary ("traffic_bytes_per_launch: N")."""
+    """(bytes per launch or None, description) of the gate/up GEMM's HBM traffic from the committed counter summary.
+
+    The summary carries "traffic_bytes_per_launch: N" and "kernel_source_sha256: H" (hash of the kernel sources the
+    counters were read on, see kernel_source_hash); a figure taken on other sources is not reported."""
     path = TRAFFIC_FILE.format(config=config_name.split("_")[0])
+    rel = os.path.relpath(path, ROOT)
+    now = kernel_source_hash()
     if not os.path.exists(path):
-        return None
+        return None, {"file": None, "kernel_source_sha256": now, "note": "no counter summary for this workload"}
+    value, taken_on = None, None
     for line in open(path):
         if line.startswith("traffic_bytes_per_launch:"):
-            return float(line.split(":", 1)[1])
-    return None
+            value = float(line.split(":", 1)[1])
+        if line.startswith("kernel_source_sha256:"):
+            taken_on = line.split(":", 1)[1].strip()
+    src = {"file": rel, "recorded_on_kernel_source_sha256": taken_on, "kernel_source_sha256": now,
+           "note": "recorded by separate rocprofv3 --pmc runs, not measured by this run"}
+    if taken_on != now:
+        src["note"] = "the counter summary was taken on other kernel sources: not reported"
+        return None, src
+    return value, src
+
+
+def _gate_up_roofline(cfg, touched, kernels):
+    """Roofline block of the gate/up grouped GEMM from the library's event timer.
+
+    Algorithmic bytes of one launch: the touched experts' gate/up weights and channel scales, the expanded int8 rows
+    and their scales in, the int8 activations and their scales out.  Algorithmic ops: 4 * M * H * I."""
+    M, H, I = cfg.tokens * cfg.top_k, cfg.hidden, cfg.inter
+    gemm1_bytes = touched * 2 * H * I + touched * 2 * I * 4 + M * H + M * 4 + M * I + M * 4
+    gemm1_ops = 4 * M * H * I
+    n1, total1 = kernels.get("gmm_swiglu", (0, 0.0))
+    gemm1_ms = total1 / max(n1, 1)
+    hbm_frac = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if gemm1_ms > 0 else None
+    mfma_frac = gemm1_ops / (gemm1_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS if gemm1_ms > 0 else None
+    # bound of the kernel at this shape: time at HBM peak vs time at MFMA peak
+    t_hbm = gemm1_bytes / (HBM_PEAK_GBS * 1e9)
+    t_mfma = gemm1_ops / (INT8_PEAK_TOPS * 1e12)
+    traffic, traffic_source = _recorded_traffic(cfg.name)
+    if t_hbm >= t_mfma:
+        roofline = {"bound": "hbm", "achieved": gemm1_bytes / (gemm1_ms * 1e-3) / 1e9 if gemm1_ms else None,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac, "traffic": traffic}
+    else:
+        roofline = {"bound": "mfma", "achieved": gemm1_ops / (gemm1_ms * 1e-3) / 1e12 if gemm1_ms else None,
+                    "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": traffic}
+    roofline.update({"traffic_source": traffic_source,
+                     "kernel": "StreamGemmKernel<..., kSwiglu> (gate/up GEMM + SwiGLU; timer name gmm_swiglu)",
+                     "kernel_ms": gemm1_ms, "algorithmic_bytes": gemm1_bytes, "algorithmic_ops": gemm1_ops,
+                     "hbm_frac": hbm_frac, "mfma_frac": mfma_frac})
+    return roofline
+
+
+class Workload:
+    """One configuration resident on the GPU: routing inputs, quantised activations, expert weights, the chain."""
+
+    def __init__(self, pkg, cfg, dev, routing="v3", **ffn_kwargs):
+        import torch
+        self.pkg, self.cfg, self.dev = pkg, cfg, dev
+        seed = pkg.synth.CONFIGS.index(cfg)
+        self.idx, self.wgt = pkg.synth.make_routing(cfg, seed=seed)
+        self.xq, self.xs = pkg.synth.make_activations(cfg, seed=seed)
+        self.weights = pkg.synth.make_weights(cfg, dev, seed=seed)
+        self.ffn_kwargs = ffn_kwargs
+        self.ffn = pkg.MoeFfnW8A8(*self.weights, routing=routing, **ffn_kwargs)
+        self.d_xq, self.d_xs = torch.from_numpy(self.xq).to(dev), torch.from_numpy(self.xs).to(dev)
+        self.d_idx, self.d_wgt = torch.from_numpy(self.idx).to(dev), torch.from_numpy(self.wgt).to(dev)
+        self.touched = int((np.bincount(self.idx.reshape(-1), minlength=cfg.experts) > 0).sum())
+
+    def with_routing(self, routing):
+        """The same tensors behind a chain that starts with another routing operator."""
+        other = object.__new__(Workload)
+        other.__dict__.update(self.__dict__)
+        other.ffn = self.pkg.MoeFfnW8A8(*self.weights, routing=routing, **self.ffn_kwargs)
+        return other
+
+    def measure(self, steps, warmup, graph=False):
+        """Times `steps` passes (after `warmup` untimed ones) between two device synchronisations.
+
+        Returns (seconds per pass, {kernel name: (launches, total ms)}) with the kernel durations from the library's
+        HIP-event timer over the timed passes.  A graph replay runs no host code of the library, so its events see
+        nothing: the per-kernel durations then come from the same number of eager passes run right after."""
+        import torch
+        aclnn = self.pkg.aclnn
+        args = (self.d_xq, self.d_xs, self.d_idx, self.d_wgt)
+        if graph:
+            g, _ = self.ffn.capture(*args)
+            step = g.replay
+        else:
+            step = lambda: self.ffn.forward(*args)
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        aclnn.kernel_timer_enable(not graph)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        if graph:
+            aclnn.kernel_timer_enable(True)
+            for _ in range(steps):
+                self.ffn.forward(*args)
+            torch.cuda.synchronize()
+        kernels = aclnn.kernel_timer_report()
+        aclnn.kernel_timer_enable(False)
+        return elapsed / steps, kernels
+
+    def summary(self, sec_per_pass, kernels, steps, launch):
+        cfg = self.cfg
+        work = self.pkg.synth.algorithmic_work(cfg, self.touched)
+        return {
+            "workload": "%s: %d tokens, H=%d, I=%d, E=%d, top-%d, %s routing" % (
+                cfg.name, cfg.tokens, cfg.hidden, cfg.inter, cfg.experts, cfg.top_k,
+                "Zipf(%.1f)" % cfg.skew if cfg.skew else "uniform random"),
+            "chain": "%s routing, SwiGLU GEMM, down GEMM, finalize" % self.ffn.routing.upper(),
+            "launch": launch,
+            "experts_touched": self.touched,
+            "ms_per_step": sec_per_pass * 1e3,
+            "tokens_per_s": cfg.tokens / sec_per_pass,
+            "end_to_end": {"mfma_frac": work["ops"] / sec_per_pass / 1e12 / INT8_PEAK_TOPS,
+                           "hbm_frac": work["bytes"] / sec_per_pass / 1e9 / HBM_PEAK_GBS,
+                           "algorithmic_ops": work["ops"], "algorithmic_bytes": work["bytes"]},
+            "kernels_ms": {k: v[1] / float(steps) for k, v in sorted(kernels.items())},
+            "roofline": _gate_up_roofline(cfg, self.touched, kernels),
+        }
+
+
+def _other_configs(pkg, dev, headline, steps, warmup):
+    """The halves of the metric that the headline configuration does not show, measured the same way."""
+    import torch
+    out = {}
+
+    def release():
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    if headline.cfg.name.startswith("c1") and headline.ffn.routing == "v3":
+        v2 = headline.with_routing("v2")
+        sec, kernels = v2.measure(steps, warmup)
+        out["c1_v2_routed"] = v2.summary(sec, kernels, steps, "eager two-phase calls")
+        del v2
+    for name in ("c3", "c2", "c4"):
+        if headline.cfg.name.startswith(name):
+            continue
+        release()
+        w = Workload(pkg, pkg.synth.config(name), dev)
+        sec, kernels = w.measure(steps, warmup)
+        out[name] = w.summary(sec, kernels, steps, "eager two-phase calls")
+        if name == "c3":
+            sec, kernels = w.measure(steps, warmup, graph=True)
+            out["c3_graph"] = w.summary(sec, kernels, steps, "HIP graph replay (kernel durations from eager passes)")
+        del w
+    release()
+    return out
 
 
 def main():
@@ -86,9 +254,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="measure the headline configuration only (profiler runs)")
     ap.add_argument("--calibration-copy", action="store_true")
     ap.add_argument("--graph", action="store_true",
                     help="replay the pass from a HIP graph (second phases only) instead of calling the operators eagerly")
+    ap.add_argument("--routing", choices=("v2", "v3"), default="v3",
+                    help="routing operator at the head of the chain: aclnnMoeInitRoutingV3 (default) or V2")
     ap.add_argument("--weight-nz", action="store_true",
                     help="give the GEMM operators FRACTAL_NZ weights ([E, N/32, K/16, 16, 32]) instead of transposed views")
     ap.add_argument("--weight-row-major", action="store_true",
@@ -110,40 +282,10 @@ def main():
     aclnn.lib()
     dev = torch.device("cuda:0")
     cfg = pkg.synth.config(args.config)
-    seed = pkg.synth.CONFIGS.index(cfg)
 
-    idx, wgt = pkg.synth.make_routing(cfg, seed=seed)
-    xq, xs = pkg.synth.make_activations(cfg, seed=seed)
-    w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=seed)
-    ffn = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, fused_combine=args.fused_combine, weight_nz=args.weight_nz,
-                         weight_row_major=args.weight_row_major)
-    d_xq, d_xs = torch.from_numpy(xq).to(dev), torch.from_numpy(xs).to(dev)
-    d_idx, d_wgt = torch.from_numpy(idx).to(dev), torch.from_numpy(wgt).to(dev)
-
-    if args.graph:
-        graph, _ = ffn.capture(d_xq, d_xs, d_idx, d_wgt)
-        step = graph.replay
-    else:
-        step = lambda: ffn.forward(d_xq, d_xs, d_idx, d_wgt)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-
-    aclnn.kernel_timer_enable(True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    if args.graph:
-        # a replay runs no host code of the library, so its event timer sees nothing: the per-kernel durations come
-        # from the same number of eager passes run right after the timed region
-        for _ in range(args.steps):
-            ffn.forward(d_xq, d_xs, d_idx, d_wgt)
-        torch.cuda.synchronize()
-    kernels = aclnn.kernel_timer_report()
-    aclnn.kernel_timer_enable(False)
+    head = Workload(pkg, cfg, dev, routing=args.routing, fused_combine=args.fused_combine, weight_nz=args.weight_nz,
+                    weight_row_major=args.weight_row_major)
+    sec_per_pass, kernels = head.measure(args.steps, args.warmup, graph=args.graph)
     if args.calibration_copy:
         src = torch.empty(1 << 30, dtype=torch.int8, device=dev).fill_(3)
         dst = torch.empty_like(src)
@@ -152,67 +294,39 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    ms_per_step = elapsed / args.steps * 1e3
-    tokens_per_s = cfg.tokens / (elapsed / args.steps)
-    counts = np.bincount(idx.reshape(-1), minlength=cfg.experts)
-    touched = int((counts > 0).sum())
-    work = pkg.synth.algorithmic_work(cfg, touched)
-    M, H, I = cfg.tokens * cfg.top_k, cfg.hidden, cfg.inter
-
-    # dominant kernel: the gate/up grouped GEMM.  Algorithmic bytes of one launch: the touched experts' gate/up weights
-    # and channel scales, the expanded int8 rows and their scales in, the int8 activations and their scales out.
-    gemm1_bytes = touched * 2 * H * I + touched * 2 * I * 4 + M * H + M * 4 + M * I + M * 4
-    gemm1_ops = 4 * M * H * I
-    n1, total1 = kernels.get("gmm_swiglu", (0, 0.0))
-    gemm1_ms = total1 / max(n1, 1)
-    hbm_frac = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if gemm1_ms > 0 else None
-    mfma_frac = gemm1_ops / (gemm1_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS if gemm1_ms > 0 else None
-    # bound of the kernel at this shape: time at HBM peak vs time at MFMA peak
-    t_hbm = gemm1_bytes / (HBM_PEAK_GBS * 1e9)
-    t_mfma = gemm1_ops / (INT8_PEAK_TOPS * 1e12)
-    if t_hbm >= t_mfma:
-        roofline = {"bound": "hbm", "achieved": gemm1_bytes / (gemm1_ms * 1e-3) / 1e9 if gemm1_ms else None,
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac, "traffic": _recorded_traffic(cfg.name)}
-    else:
-        roofline = {"bound": "mfma", "achieved": gemm1_ops / (gemm1_ms * 1e-3) / 1e12 if gemm1_ms else None,
-                    "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": _recorded_traffic(cfg.name)}
-    roofline.update({"kernel": "StreamGemmKernel<..., kSwiglu> (gate/up GEMM + SwiGLU; timer name gmm_swiglu)", "kernel_ms": gemm1_ms,
-                     "algorithmic_bytes": gemm1_bytes, "algorithmic_ops": gemm1_ops,
-                     "hbm_frac": hbm_frac, "mfma_frac": mfma_frac})
-
+    s = head.summary(sec_per_pass, kernels, args.steps, "HIP graph replay" if args.graph else "eager two-phase calls")
+    work = pkg.synth.algorithmic_work(cfg, head.touched)
     result = {
         "metric": "MoE FFN tokens/s (W8A8 expert FFN: routing + gate/up GEMM + SwiGLU + requant + down GEMM + finalize), 1 GPU",
-        "value": tokens_per_s,
+        "value": s["tokens_per_s"],
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": s["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "int8",
         "data": "synthetic",
-        "config": {"workload": "%s: %d tokens, H=%d, I=%d, E=%d, top-%d, %s routing" % (
-            cfg.name, cfg.tokens, cfg.hidden, cfg.inter, cfg.experts, cfg.top_k,
-            "Zipf(%.1f)" % cfg.skew if cfg.skew else "uniform random"),
-            "expanded_rows": M, "experts_touched": touched, "weight_layout": "FRACTAL_NZ" if args.weight_nz else "row-major [E, K, N]" if args.weight_row_major
-            else "K-contiguous (transposed view)",
-            "chain": "V3 routing, SwiGLU GEMM, " + ("fused down GEMM + combine" if args.fused_combine else "down GEMM, finalize"),
-            "launch": "HIP graph replay" if args.graph else "eager two-phase calls"},
-        "end_to_end": {"tops": work["ops"] / (elapsed / args.steps) / 1e12, "gbps": work["bytes"] / (elapsed / args.steps) / 1e9,
-                       "mfma_frac": work["ops"] / (elapsed / args.steps) / 1e12 / INT8_PEAK_TOPS,
-                       "hbm_frac": work["bytes"] / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,
-                       "algorithmic_ops": work["ops"], "algorithmic_bytes": work["bytes"]},
-        "kernels_ms": {k: v[1] / max(v[0], 1) * (v[0] / float(args.steps)) for k, v in sorted(kernels.items())},
-        "roofline": roofline,
+        "config": {"workload": s["workload"], "expanded_rows": cfg.tokens * cfg.top_k, "experts_touched": head.touched,
+                   "weight_layout": "FRACTAL_NZ" if args.weight_nz else "row-major [E, K, N]" if args.weight_row_major
+                   else "K-contiguous (transposed view)",
+                   "chain": "%s routing, SwiGLU GEMM, " % args.routing.upper() +
+                            ("fused down GEMM + combine" if args.fused_combine else "down GEMM, finalize"),
+                   "launch": s["launch"]},
+        "end_to_end": dict(s["end_to_end"], tops=work["ops"] / sec_per_pass / 1e12, gbps=work["bytes"] / sec_per_pass / 1e9),
+        "kernels_ms": s["kernels_ms"],
+        "roofline": s["roofline"],
     }
     if not args.no_cpu_baseline:
         oracle = graft.load_oracle()
         oracle.build()
-        v, desc = _cpu_baseline(pkg, oracle, cfg, idx, wgt, xq, xs, ffn)
+        v, desc = _cpu_baseline(pkg, oracle, cfg, head.idx, head.wgt, head.xq, head.xs, head.ffn)
         result["cpu_baseline"] = {"value": v, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
                                   "sample": desc}
+    if not args.no_other_configs:
+        result["other_configs"] = _other_configs(pkg, dev, head, steps=min(args.steps, 10), warmup=min(args.warmup, 2))
     print(json.dumps(result))
 
 

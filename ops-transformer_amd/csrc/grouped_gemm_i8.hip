@@ -1107,8 +1107,10 @@ bool StreamOk(const Problem& p) {
     const int64_t grain = p.wNz ? 32 : 16;
     const bool layoutOk = p.wKMajor && !p.wNz ? true
                           : (p.N % grain == 0 && (p.epilogue != Epilogue::kSwiglu || (p.N / 2) % grain == 0));
+    // One expert's weights must hold at least the kilobyte (64 lanes x 16 bytes) that a drained workgroup's idle issue
+    // slots keep re-reading from the start of its last tile's expert: smaller experts go to the byte-wise kernel.
     return layoutOk && p.K % 128 == 0 && reinterpret_cast<uintptr_t>(p.x) % kChunk == 0 &&
-           reinterpret_cast<uintptr_t>(p.w) % kChunk == 0 && p.N * p.K < (1ll << 31);
+           reinterpret_cast<uintptr_t>(p.w) % kChunk == 0 && p.N * p.K < (1ll << 31) && p.N * p.K >= 64 * kChunk;
 }
 
 uint64_t Align256(uint64_t v) { return (v + 255) / 256 * 256; }

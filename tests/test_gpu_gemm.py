@@ -38,6 +38,10 @@ def _weight_views(wt, dev, layout):
 INT32_CASES = [  # M, K, N, E, mode, layout
     (1, 16, 8, 1, "even", "kmajor"),
     (37, 128, 24, 4, "ragged", "kmajor"),
+    (37, 128, 2, 4, "ragged", "kmajor"),         # one expert's weights are shorter than a kilobyte: byte-wise loader
+    (64, 384, 2, 3, "even", "kmajor"),
+    (37, 128, 6, 4, "ragged", "kmajor"),
+    (37, 128, 8, 4, "ragged", "kmajor"),         # exactly one kilobyte per expert: the ring kernel
     (96, 256, 300, 7, "ragged", "kmajor"),
     (512, 1024, 512, 8, "even", "kmajor"),       # tile 96
     (512, 4096, 256, 128, "ragged", "kmajor"),   # decode-like: tile 32, many groups

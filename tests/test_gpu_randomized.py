@@ -94,7 +94,7 @@ def test_grouped_gemm_random(aclnn, oracle, dev, seed):
     rng = np.random.default_rng(3000 + seed)
     M = int(rng.integers(1, 700))
     K = int(rng.choice([16, 48, 128, 200, 256, 384, 1024]))
-    N = int(rng.choice([8, 64, 96, 256, 264, 512]))
+    N = int(rng.choice([2, 4, 8, 64, 96, 256, 264, 512]))
     E = int(rng.choice([1, 2, 5, 16, 40]))
     x = rng.integers(-127, 128, (M, K)).astype(np.int8)
     wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
