@@ -29,6 +29,19 @@ ACLNN_API aclnnStatus aclnnMoeInitRoutingV2GetWorkspaceSize(
 ACLNN_API aclnnStatus aclnnMoeInitRoutingV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
                                             aclrtStream stream);
 
+/*
+ * aclnnMoeInitRoutingV2StaticWorkspace -- no counterpart in the reference.  For callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the second phase of
+ * aclnnMoeInitRoutingV2 without a workspace argument.  The sort tables live in a 4 MiB device array inside the library
+ * (one copy per GPU, held until the process ends), which covers up to about 130000 expanded rows (tokens x top-k) per call with expertNum <= 2048.
+ * Takes an executor made by aclnnMoeInitRoutingV2GetWorkspaceSize and consumes it like the ordinary second phase; a call
+ * whose first phase asked for more than 4 MiB is refused with ACLNN_ERR_PARAM_INVALID (the executor is released).  Calls
+ * no hipMalloc / hipFree.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
+ * race -- serialise them.  The first call on a device looks the array's address up (hipGetSymbolAddress), so make one
+ * call before starting a graph capture.
+ */
+ACLNN_API aclnnStatus aclnnMoeInitRoutingV2StaticWorkspace(aclOpExecutor* executor, aclrtStream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -108,6 +108,8 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = [_VP, ctypes.c_uint64, _VP, _VP]
             fn.restype = ctypes.c_int32
+        l.aclnnMoeInitRoutingV2StaticWorkspace.argtypes = [_VP, _VP]
+        l.aclnnMoeInitRoutingV2StaticWorkspace.restype = ctypes.c_int32
         l.aclCreateTensor.argtypes = [ctypes.POINTER(_I64), ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(_I64), _I64,
                                       ctypes.c_int, ctypes.POINTER(_I64), ctypes.c_uint64, _VP]
         l.aclCreateTensor.restype = _VP
@@ -218,14 +220,22 @@ def _stream_ptr():
     return torch.cuda.current_stream().cuda_stream
 
 
-def _run_two_phase(api, args, device, workspace=None):
-    """args: phase-1 arguments without the two trailing out-parameters."""
+def _run_two_phase(api, args, device, workspace=None, static_workspace_api=None):
+    """args: phase-1 arguments without the two trailing out-parameters.
+
+    static_workspace_api names a second phase that takes (executor, stream) only and keeps its scratch inside the
+    library: no workspace is allocated or passed."""
     l = lib()
     ws_size = ctypes.c_uint64(0)
     executor = ctypes.c_void_p(None)
     st = getattr(l, api + "GetWorkspaceSize")(*args, ctypes.byref(ws_size), ctypes.byref(executor))
     if st != ACLNN_SUCCESS:
         raise AclnnError(api + "GetWorkspaceSize", st, last_error())
+    if static_workspace_api is not None:
+        st = getattr(l, static_workspace_api)(executor, _VP(_stream_ptr()))
+        if st != ACLNN_SUCCESS:
+            raise AclnnError(static_workspace_api, st, last_error())
+        return None
     ws_ptr = None
     ws_keepalive = None
     if ws_size.value > 0:
@@ -255,9 +265,11 @@ def workspace_size(api, args):
 # ------------------------------------------------------------------------------------------------ operators
 def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_num=0, drop_pad_mode=0,
                         expert_tokens_count_or_cumsum_flag=0, expert_tokens_before_capacity_flag=False, out=None,
-                        workspace=None):
+                        workspace=None, static_workspace=False):
     """aclnnMoeInitRoutingV2.  Returns (expanded_x, expanded_row_idx, expert_tokens_count_or_cumsum | None,
-    expert_tokens_before_capacity | None).  ``out`` may carry preallocated outputs in that order."""
+    expert_tokens_before_capacity | None).  ``out`` may carry preallocated outputs in that order.
+    static_workspace=True runs the second phase through aclnnMoeInitRoutingV2StaticWorkspace (no device allocation;
+    with ``out`` given the call allocates nothing on the device at all)."""
     T, H = x.shape
     K = expert_idx.shape[1]
     M = T * K
@@ -280,7 +292,8 @@ def moe_init_routing_v2(x, expert_idx, active_num=0, expert_capacity=0, expert_n
         args = [h.tensor(x), h.tensor(expert_idx), active_num, expert_capacity, expert_num, drop_pad_mode,
                 expert_tokens_count_or_cumsum_flag, bool(expert_tokens_before_capacity_flag), h.tensor(expanded_x),
                 h.tensor(expanded_row_idx), h.tensor(count_out), h.tensor(before_out)]
-        _run_two_phase("aclnnMoeInitRoutingV2", args, dev, workspace)
+        _run_two_phase("aclnnMoeInitRoutingV2", args, dev, workspace,
+                       static_workspace_api="aclnnMoeInitRoutingV2StaticWorkspace" if static_workspace else None)
     finally:
         h.close()
     return expanded_x, expanded_row_idx, count_out, before_out

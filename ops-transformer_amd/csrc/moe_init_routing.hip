@@ -24,6 +24,8 @@
 
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "aclnnop/aclnn_moe_init_routing_quant_v2.h"
 #include "aclnnop/aclnn_moe_init_routing_v2.h"
 #include "aclnnop/aclnn_moe_init_routing_v3.h"
@@ -1053,6 +1055,72 @@ extern "C" aclnnStatus aclnnMoeInitRoutingQuantV2(void* workspace, uint64_t work
 extern "C" aclnnStatus aclnnMoeInitRoutingV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
                                              aclrtStream stream) {
     return opapi::RunAndRelease(workspace, workspaceSize, executor, stream);
+}
+
+// ---------------------------------------------------------------------------------------------- allocation-free second phase
+// aclnnMoeInitRoutingV2StaticWorkspace: the second phase of aclnnMoeInitRoutingV2 for callers that cannot allocate
+// device memory (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The sort tables that
+// the ordinary second phase keeps in the caller's workspace live in a file-scope device array instead; every GPU the
+// library runs on holds its own copy of the array until the process ends.
+constexpr uint64_t kStaticScratchBytes = 4ull << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxScratchDevices = 64;
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a stand-in for the symbol:
+// the address that kernels can use comes from hipGetSymbolAddress, asked once per device with that device current.
+hipError_t StaticScratchOfCurrentDevice(void** out) {
+    static std::mutex mu;
+    static void* ptrOfDevice[kMaxScratchDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxScratchDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptrOfDevice[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        ptrOfDevice[dev] = p;
+    }
+    *out = ptrOfDevice[dev];
+    return hipSuccess;
+}
+
+}  // namespace
+
+extern "C" aclnnStatus aclnnMoeInitRoutingV2StaticWorkspace(aclOpExecutor* executor, aclrtStream stream) {
+    opapi::ClearError();
+    if (executor == nullptr) {
+        opapi::SetError("aclnnMoeInitRoutingV2StaticWorkspace: executor must not be null");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    const InitRoutingExecutor* const routing = dynamic_cast<const InitRoutingExecutor*>(executor);
+    if (routing == nullptr || routing->v3 || routing->dynamicQuant || routing->staticScale != nullptr) {
+        opapi::SetError("aclnnMoeInitRoutingV2StaticWorkspace: the executor was not made by aclnnMoeInitRoutingV2GetWorkspaceSize");
+        delete executor;
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    if (executor->workspaceBytes > kStaticScratchBytes) {
+        opapi::SetError("aclnnMoeInitRoutingV2StaticWorkspace: this call needs %llu bytes of workspace, the built-in scratch "
+                        "area holds %llu: use aclnnMoeInitRoutingV2 with a caller-provided workspace",
+                        (unsigned long long)executor->workspaceBytes, (unsigned long long)kStaticScratchBytes);
+        delete executor;
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    void* ptr = nullptr;
+    const hipError_t e = StaticScratchOfCurrentDevice(&ptr);
+    if (e != hipSuccess) {
+        opapi::SetError("aclnnMoeInitRoutingV2StaticWorkspace: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        delete executor;
+        return ACLNN_ERR_RUNTIME_ERROR;
+    }
+    // Nothing in the sort tables has to start at zero (every kernel writes what the next one reads), so the contents
+    // left by the previous call need no clearing.
+    return opapi::RunAndRelease(ptr, kStaticScratchBytes, executor, stream);
 }
 
 // ---------------------------------------------------------------------------------------------- aclnnMoeInitRoutingV3
