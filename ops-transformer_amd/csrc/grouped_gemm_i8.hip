@@ -543,7 +543,7 @@ struct StreamCfg {
     static_assert(kTileM % kRowsPerInstr == 0, "tile rows must fill whole DMA instructions");
     static constexpr int kMaxPerWave = (kInstr + kWaves - 1) / kWaves;
     static_assert(kStages >= 2, "the ring needs at least two stages");
-    static_assert((kStages - 2) * kMaxPerWave <= 63, "vmcnt is a 6-bit counter");
+    static_assert((kStages - 1) * kMaxPerWave <= 63, "vmcnt is a 6-bit counter");
 };
 
 // Byte offset of 16-byte chunk `chunk` of row `row` in a stage whose rows are kStep bytes.  The LDS serves 16 lanes per
@@ -704,7 +704,8 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             }
         }
     };
-    auto issueStage = [&](int ring) __attribute__((always_inline)) {
+    // DMA instruction q (0 .. kMaxPerWave - 1) of this wave's share of the stage at the issue cursor, into buffer `ring`.
+    auto issueOne = [&](int ring, int q) __attribute__((always_inline)) {
         const uint32_t dst = ldsBase + ring * kStageBytes;
         // On small tiles the k-steps of a tile are walked from a start that differs between workgroups (integer
         // accumulation does not care about the order).  When rows lie a power-of-two stride apart (K = 4096 with
@@ -716,19 +717,19 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         const int kOff = issDrained ? 0 : (kIdx >= kSteps ? kIdx - kSteps : kIdx) * kStep;
         // blocked layout: one k is 32 bytes further; row-major: N bytes
         const int kOffW = kNz ? kOff * 32 : (kNMajor ? kOff * a.N : kOff);
-#pragma unroll
-        for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
-            const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
-            // wave-uniform branch: activation rows always stay cacheable (the n-tiles of a group re-read them from L2);
-            // on small tiles (every weight byte is used exactly once) the weights stream past the caches.  On large
-            // tiles the m-tiles of a group share their weight columns through L2 and must not.
-            if constexpr (kSmallTile) {
-                if (j < Cfg::kInstrA) DmaToLdsAddr16<false>(issX + kOff, laneOff[q], dst + j * 1024);
-                else DmaToLdsAddr16<true>(issW + kOffW, laneOff[q], dst + j * 1024);
-            } else {
-                DmaToLdsAddr16<false>(j < Cfg::kInstrA ? issX + kOff : issW + kOffW, laneOff[q], dst + j * 1024);
-            }
+        const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
+        // wave-uniform branch: activation rows always stay cacheable (the n-tiles of a group re-read them from L2);
+        // on small tiles (every weight byte is used exactly once) the weights stream past the caches.  On large
+        // tiles the m-tiles of a group share their weight columns through L2 and must not.
+        if constexpr (kSmallTile) {
+            if (j < Cfg::kInstrA) DmaToLdsAddr16<false>(issX + kOff, laneOff[q], dst + j * 1024);
+            else DmaToLdsAddr16<true>(issW + kOffW, laneOff[q], dst + j * 1024);
+        } else {
+            DmaToLdsAddr16<false>(j < Cfg::kInstrA ? issX + kOff : issW + kOffW, laneOff[q], dst + j * 1024);
         }
+    };
+    // Moves the issue cursor to the next k-step (after the last instruction of a stage has gone out).
+    auto issueAdvance = [&]() __attribute__((always_inline)) {
         if (++issStep == kSteps) {
             // move to this workgroup's next tile.  Past the last one the issue slots still go out (that keeps the number
             // of outstanding DMAs per stage, hence the vmcnt arithmetic, constant) into ring slots nobody reads -- but
@@ -749,10 +750,28 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         }
     };
 
+    // A whole stage at once: every instruction of this wave's share, then the cursor moves on.
+    auto issueStage = [&](int ring) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < Cfg::kMaxPerWave; ++q) issueOne(ring, q);
+        issueAdvance();
+    };
+
+    // Shifted barrier (tall tiles).  The plain k-step opens with its barrier -- the stage has landed, the previous one is
+    // no longer read -- after which every wave waits for its first fragments before it has any MFMA to issue.  Here the
+    // step's one barrier sits in front of its LAST block of MFMAs instead: by then every k-slice of the stage has been
+    // read, so the buffer takes its refill a quarter of a step earlier, the same barrier certifies the next stage as
+    // landed, and the next step's first fragments are read while the matrix pipe still has a block of MFMAs to run.  All
+    // kStages buffers are in use.
+    constexpr bool kEarly = kTileM >= 96;
     setupIssue();
 #pragma unroll 1
-    for (int s = 0; s < kStages - 1; ++s) issueStage(s);
-    int ring = 0;  // stage the compute side reads next; the issue side writes (ring + kStages - 1) % kStages
+    for (int s = 0; s < (kEarly ? kStages : kStages - 1); ++s) issueStage(s);
+    int ring = 0;  // stage the compute side reads next; the issue side writes (ring + kStages - 1) % kStages (kEarly: ring itself)
+    if constexpr (kEarly) {
+        WaitVmcnt<(kStages - 1) * Cfg::kMaxPerWave>();
+        __syncthreads();  // stage 0 has landed for every wave
+    }
 
     if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
         ldsRowScale[tid] = a.rowScale[cur.rowBase + (tid < cur.rows ? tid : cur.rows - 1)];
@@ -782,25 +801,28 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
 
-        // One k-step of a wave with kMy MFMA tiles: straight-line code, the operands of k-slice ks + 1 are read
-        // from LDS before the MFMAs of k-slice ks are issued, and the refill of the stage freed by the barrier goes out
-        // behind the first block of MFMAs (its scalar address work then runs in the shadow of the matrix pipe).
-        auto computeStep = [&](auto myTag) __attribute__((always_inline)) {
+        // The k loop of a wave with kMy MFMA tiles.  A k-step is straight-line code: the operands of k-slice ks + 1 are
+        // read from LDS before the MFMAs of k-slice ks are issued (fragment double buffer af / bf).
+        // Plain form: one barrier at the start of a step (the stage has landed, the previous one is no longer read),
+        // and the refill of the buffer it frees goes out behind the first block of MFMAs.
+        // kEarly form: see above; the fragments of a step's first k-slice are read at the end of the step before.
+        auto runTile = [&](auto myTag) __attribute__((always_inline)) {
             constexpr int kMy = decltype(myTag)::value;
-            const char* const A = lds + ring * kStageBytes;
-            const char* const B = A + kTileM * kStep;
             constexpr int kSlices = kStep / 32;
+            static_assert(kSlices % 2 == 0, "the fragment double buffer is handed over between steps at slot 0");
             v4i bf[2][2];
             v4i af[2][kMy > 0 ? kMy : 1];
-            auto loadSlice = [&](int ks, int buf) __attribute__((always_inline)) {
+            auto loadSlice = [&](int stage, int ks, int buf) __attribute__((always_inline)) {
                 if (kMy == 0) return;
+                const char* const A = lds + stage * kStageBytes;
+                const char* const B = A + kTileM * kStep;
                 const int chunk = 2 * ks + lhi;
                 if constexpr (kNMajor) {
                     // 16-lane group g: channels 16 * (g % 2) .. + 15 of the 32-channel block, k-half g / 2 (= lhi) of the
                     // slice; lane j of the group supplies bytes (k = kBase + j / 2, channels 8 * (j % 2) .. + 7)
                     const int j = lane & 15;
                     const int k = 32 * ks + 16 * lhi + (j >> 1);
-                    const uint32_t bBase = ldsBase + ring * kStageBytes + kTileM * kStep + 8 * (j & 1);
+                    const uint32_t bBase = ldsBase + stage * kStageBytes + kTileM * kStep + 8 * (j & 1);
 #pragma unroll
                     for (int ni = 0; ni < 2; ++ni) {
                         const int c = (bRow0 + ni * bRowStep + 16 * ((lane >> 4) & 1)) >> 4;  // logical 16-byte chunk of the row
@@ -819,7 +841,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
 #pragma unroll
                     for (int ni = 0; ni < 2; ++ni) {
                         // addressed through the 32-bit LDS address: no generic-to-LDS pointer conversion in the loop
-                        const uint32_t blk = ldsBase + ring * kStageBytes + kTileM * kStep +
+                        const uint32_t blk = ldsBase + stage * kStageBytes + kTileM * kStep +
                                              ((bRow0 + ni * bRowStep) >> 5) * 4096 + inBlock;
                         const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk));
                         const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk + 8 * 32));
@@ -834,27 +856,39 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                     af[buf][mi] = *reinterpret_cast<const v4i*>(A + LdsOffset<kStep>(waveRow0 + mi * 32 + l32, chunk));
                 }
             };
-            loadSlice(0, 0);
-#pragma unroll
-            for (int ks = 0; ks < kSlices; ++ks) {
-                if (ks + 1 < kSlices) loadSlice(ks + 1, (ks + 1) & 1);
-#pragma unroll
-                for (int mi = 0; mi < kMy; ++mi) {
-                    acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][0], acc[mi][0], 0, 0, 0);
-                    acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][1], acc[mi][1], 0, 0, 0);
-                }
-                if (ks == 0) issueStage(ring == 0 ? kStages - 1 : ring - 1);
-            }
-        };
-
-        auto runTile = [&](auto myTag) __attribute__((always_inline)) {
+            if constexpr (kEarly) loadSlice(ring, 0, 0);  // the tile's first stage was certified at the end of the tile before
 #pragma unroll 1
             for (int step = 0; step < kSteps; ++step) {
-                // the oldest stage in flight has landed once at most (kStages - 2) stages' worth of this wave's DMAs remain
-                WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
-                __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
-                computeStep(myTag);
-                ring = ring + 1 == kStages ? 0 : ring + 1;
+                if constexpr (!kEarly) {
+                    // the oldest stage in flight has landed once at most (kStages - 2) stages' worth of this wave's DMAs remain
+                    WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
+                    __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
+                    loadSlice(ring, 0, 0);
+                }
+                const int nextRing = ring + 1 == kStages ? 0 : ring + 1;
+#pragma unroll
+                for (int ks = 0; ks < kSlices; ++ks) {
+                    if (!kEarly || ks + 1 < kSlices) {
+                        if (ks + 1 < kSlices) loadSlice(ring, ks + 1, (ks + 1) & 1);
+                    } else {
+                        // Before the step's last block of MFMAs: every k-slice of this stage has been read (the reads
+                        // of the last one returned in the shadow of the block before), and the next stage, issued one
+                        // step ago, should have landed.  One barrier certifies both; inside a tile, the next step's
+                        // first fragments are read behind the MFMAs.
+                        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads have returned
+                        WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
+                        __syncthreads();
+                        issueStage(ring);
+                        if (step + 1 < kSteps) loadSlice(nextRing, 0, 0);
+                    }
+#pragma unroll
+                    for (int mi = 0; mi < kMy; ++mi) {
+                        acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][0], acc[mi][0], 0, 0, 0);
+                        acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][1], acc[mi][1], 0, 0, 0);
+                    }
+                    if (!kEarly && ks == 0) issueStage(ring == 0 ? kStages - 1 : ring - 1);
+                }
+                ring = nextRing;
             }
         };
         {
