@@ -147,6 +147,91 @@ __global__ __launch_bounds__(256) void FinalizeKernel(FinalizeArgs a, int scaleI
     }
 }
 
+// The common case -- no bias, at most kMaxK experts per token, 16-byte packets, one packet per lane -- with every load of a
+// token's K row indices and weights loaded up front (wave-uniform loads) and the K row packets requested two at a time,
+// one pair ahead of the sum, which runs in ascending k with the same separate multiply and add as the general kernel
+// (bit-identical results).  The general kernel makes 2 K dependent memory round trips per lane, this one K / 2 + 1.
+template <typename Codec, int kVec, int kMaxK>
+__global__ __launch_bounds__(256) void FinalizeBatchedKernel(FinalizeArgs a, int scaleIsF32) {
+    using P = Packet<Codec, kVec>;
+    // consecutive workgroups take the slices of one token: neighbouring pieces of the same K rows are read together
+    const int64_t packets = a.hidden / kVec;
+    const int64_t slices = (packets + 255) / 256;
+    const int64_t token = blockIdx.x / slices;
+    const int64_t pk = (blockIdx.x % slices) * 256 + threadIdx.x;
+    if (pk >= packets) return;
+    const bool columnArrangement = a.dropPadMode == 0 || a.dropPadMode == 1;
+    const bool skipsAllowed = a.dropPadMode == 1 || a.dropPadMode == 3;
+    constexpr int dataIsF16 = Codec::kRoundEveryOp ? 1 : 0;
+    const int topK = a.topK;
+
+    int64_t d[kMaxK];
+    float s[kMaxK];
+#pragma unroll
+    for (int k = 0; k < kMaxK; ++k) {
+        d[k] = -1;
+        s[k] = 1.0f;
+        if (k < topK) {
+            d[k] = columnArrangement ? a.expandedRowIdx[static_cast<int64_t>(k) * a.tokens + token]
+                                     : a.expandedRowIdx[token * topK + k];
+            if (a.scales != nullptr) s[k] = ScaleAt(a.scales, token * topK + k, scaleIsF32, dataIsF16);
+        }
+    }
+    P p1{}, p2{};
+    if (a.x1 != nullptr) p1 = static_cast<const P*>(a.x1)[token * packets + pk];
+    if (a.x2 != nullptr) p2 = static_cast<const P*>(a.x2)[token * packets + pk];
+    // row packets travel in pairs, the next pair requested before the current one is added
+    P row[2][2];
+    auto request = [&](int k0, int slot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int k = k0 + j;
+            const bool valid = k < kMaxK && k < topK && d[k < kMaxK ? k : 0] >= 0 && d[k < kMaxK ? k : 0] < a.expandedRows;
+            if (valid) row[slot][j] = static_cast<const P*>(a.expandedX)[d[k] * packets + pk];
+        }
+    };
+    request(0, 0);
+    float acc[kVec];
+    bool init = false;
+    if (a.x1 != nullptr && a.x2 != nullptr) {
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) acc[i] = Codec::Round(__fadd_rn(Codec::Load(p1.v[i]), Codec::Load(p2.v[i])));
+        init = true;
+    } else if (a.x1 != nullptr || a.x2 != nullptr) {
+        const P& only = a.x1 != nullptr ? p1 : p2;
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) acc[i] = __fadd_rn(Codec::Load(only.v[i]), 0.0f);
+        init = true;
+    }
+#pragma unroll
+    for (int k0 = 0; k0 < kMaxK; k0 += 2) {
+        if (k0 + 2 < kMaxK) request(k0 + 2, ((k0 >> 1) + 1) & 1);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int k = k0 + j;
+            if (k >= topK) continue;
+            if (d[k] < 0 || d[k] >= a.expandedRows) {
+                if (skipsAllowed && !init) {
+#pragma unroll
+                    for (int i = 0; i < kVec; ++i) acc[i] = 0.0f;
+                    init = true;
+                }
+                continue;
+            }
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                const float t = Codec::Round(__fmul_rn(Codec::Load(row[(k0 >> 1) & 1][j].v[i]), s[k]));
+                acc[i] = init ? Codec::Round(__fadd_rn(acc[i], t)) : t;
+            }
+            init = true;
+        }
+    }
+    P o;
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) o.v[i] = Codec::Store(init ? acc[i] : 0.0f);
+    static_cast<P*>(a.out)[token * packets + pk] = o;
+}
+
 class FinalizeExecutor : public aclOpExecutor {
    public:
     FinalizeArgs args{};
@@ -157,6 +242,12 @@ class FinalizeExecutor : public aclOpExecutor {
     template <typename Codec, int kVec>
     void Launch(hipStream_t stream) {
         const int64_t packets = args.hidden / kVec;
+        if (kVec > 1 && args.bias == nullptr && args.topK <= 8 && packets > 64) {
+            const unsigned slices = static_cast<unsigned>((packets + 255) / 256);
+            hipLaunchKernelGGL((FinalizeBatchedKernel<Codec, kVec, 8>), dim3(static_cast<unsigned>(args.tokens * slices)),
+                               dim3(256), 0, stream, args, scaleIsF32);
+            return;
+        }
         if (packets <= 64) {
             const unsigned blocks = static_cast<unsigned>((args.tokens + 3) / 4);
             hipLaunchKernelGGL((FinalizeKernel<Codec, kVec, 64>), dim3(blocks), dim3(256), 0, stream, args, scaleIsF32);
