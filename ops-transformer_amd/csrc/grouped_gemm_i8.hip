@@ -1200,6 +1200,9 @@ Plan MakePlan(const Problem& p) {
 hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStream_t stream) {
     if (p.M == 0 || p.N == 0 || p.groups == 0) return hipSuccess;
     if (p.groups > kMaxGroups) return hipErrorInvalidValue;
+    // K = 0 leaves the other epilogues nothing to do; with kSwiglu it would leave the requantisation an unwritten S
+    // (the operator's first phase refuses K = 0, so this is a guard, not a path)
+    if (p.K <= 0 && p.epilogue == Epilogue::kSwiglu) return hipErrorInvalidValue;
     char* ws = static_cast<char*>(workspace);
     int32_t* sched = reinterpret_cast<int32_t*>(ws + plan.offSched);
     const bool swiglu = p.epilogue == Epilogue::kSwiglu;

@@ -102,6 +102,31 @@ def test_unknown_expert_range(aclnn, oracle, dev):
     assert np.array_equal(ri, ri_r) and np.array_equal(ex, ex_r)
 
 
+@pytest.mark.parametrize("E", [200, 256])
+def test_expert_ids_outside_the_range_stay_in_bounds(aclnn, dev, E):
+    """Ids outside [0, expertNum) are undefined in the reference (its sort keys and count table assume the range).  Here
+    they give unspecified rows and counts but never an access outside the tensors: every output is guarded, the index
+    output is still a permutation of the expanded rows, and the rows written are rows of x."""
+    rng = np.random.default_rng(14)
+    T, K, H = 300, 4, 16
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    idx[rng.random((T, K)) < 0.1] = E + 3
+    idx[0, 0], idx[1, 1], idx[2, 2] = -1, 2 ** 31 - 1, -2 ** 31
+    x = rng.integers(-100, 100, (T, H)).astype(np.int8)
+    M = T * K
+    guard = 64
+    ex = torch.full((M + guard, H), 101, dtype=torch.int8, device=dev)
+    ri = torch.full((M + guard,), -7, dtype=torch.int32, device=dev)
+    cnt = torch.full((E + guard,), -7, dtype=torch.int32, device=dev)
+    aclnn.moe_init_routing_v2(torch.from_numpy(x).to(dev), torch.from_numpy(idx).to(dev), 0, 0, E, 0, 1, False,
+                              out=(ex[:M], ri[:M], cnt[:E], None))
+    torch.cuda.synchronize()
+    assert (ex[M:] == 101).all() and (ri[M:] == -7).all() and (cnt[E:] == -7).all()
+    assert np.array_equal(np.sort(ri[:M].cpu().numpy()), np.arange(M))
+    got = ex[:M].cpu().numpy()
+    assert np.array_equal(got[ri[:M].cpu().numpy()], np.repeat(x, K, axis=0))
+
+
 def test_many_experts_counts(aclnn, oracle, dev):
     """More than 2048 experts: two digit passes, counts from the sorted keys."""
     rng = np.random.default_rng(12)

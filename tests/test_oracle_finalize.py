@@ -101,6 +101,42 @@ def test_dropped_rows_contribute_nothing(oracle):
     assert (got[0] == 0).all()
 
 
+def test_dropped_rows_add_no_bias_either(oracle):
+    """Drop/pad arrangements with a bias: a dropped row (index -1) contributes NOTHING, not even scale * bias[expert].
+
+    The reference is not of one mind here.  Its bf16 and double-buffered fp kernels skip the whole term
+    (moe/moe_finalize_routing_v2/op_kernel/moe_finalize_routing_v2_bf16.h:361-366, ..._fp_db.h), while its cut-H kernels and
+    the golden of its kernel test zero the row but still add the weighted bias
+    (tests/ut/op_kernel/finalize_routing_v2_data/gen_data.py:52-59).  This build follows the former; the explicit formula
+    below pins that choice so that a change is deliberate."""
+    rng = np.random.default_rng(13)
+    T, K, H, E, C = 9, 4, 8, 5, 3
+    ex = rng.standard_normal((E, C, H)).astype(np.float32)
+    bias = rng.standard_normal((E, H)).astype(np.float32)
+    scales = rng.standard_normal((T, K)).astype(np.float32)
+    expert_idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    idx = rng.integers(0, E * C, T * K).astype(np.int32)
+    idx[rng.random(T * K) < 0.4] = -1
+    idx[:K] = -1
+    for mode in (1, 3):
+        d = idx.reshape(T, K) if mode == 3 else idx.reshape(K, T).T
+        want = np.zeros((T, H), np.float32)
+        for n in range(T):
+            for k in range(K):
+                if d[n, k] == -1:
+                    continue  # no row, no bias
+                v = (ex.reshape(-1, H)[d[n, k]] + bias[expert_idx[n, k]]).astype(np.float32)
+                want[n] = (want[n] + (v * scales[n, k]).astype(np.float32)).astype(np.float32)
+        got = oracle.moe_finalize_routing_v2(ex, idx, None, None, bias, scales, expert_idx, drop_pad_mode=mode)
+        assert np.array_equal(got, want)
+        other = want.copy()  # the reading this build does NOT follow differs on these inputs
+        for n in range(T):
+            for k in range(K):
+                if d[n, k] == -1:
+                    other[n] += bias[expert_idx[n, k]] * scales[n, k]
+        assert not np.allclose(other, want)
+
+
 @pytest.mark.parametrize("scale_f32", [True, False])
 def test_bf16_accumulates_in_fp32_and_rounds_once(oracle, scale_f32):
     rng = np.random.default_rng(12)
