@@ -202,6 +202,11 @@ class Workload:
         elapsed_timer = time.perf_counter() - t0
         kernels = aclnn.kernel_timer_report()
         aclnn.kernel_timer_enable(False)
+        # how evenly the static deal of GEMM tiles ends on the eight XCDs: one more pass with span recording on
+        aclnn.gemm_workgroup_spans_enable(True)
+        self.ffn.forward(*args)
+        self.spans = aclnn.gemm_workgroup_spans_report()
+        aclnn.gemm_workgroup_spans_enable(False)
         return elapsed / steps, kernels, elapsed_timer / steps
 
     def summary(self, measured, steps, launch):
@@ -223,7 +228,22 @@ class Workload:
                            "algorithmic_ops": work["ops"], "algorithmic_bytes": work["bytes"]},
             "kernels_ms": {k: v[1] / float(steps) for k, v in sorted(kernels.items())},
             "roofline": _gate_up_roofline(cfg, self.touched, kernels),
+            "gemm_tile_balance": self._tile_balance(),
         }
+
+    def _tile_balance(self):
+        """Per GEMM kernel: span of the launch and, over the eight XCDs, when the last workgroup of each ended and the
+        mean busy fraction of its workgroups (1.0 = every workgroup worked from the first start to the last end)."""
+        out = {}
+        for name, rec in sorted(getattr(self, "spans", {}).items()):
+            ends = [x["end_us"] for x in rec["xcd"]]
+            out[name] = {"span_us": rec["span_us"], "tile_rows": rec["tile_rows"],
+                         "xcd_end_us_min": min(ends), "xcd_end_us_max": max(ends),
+                         "xcd_busy_min": min(x["busy"] for x in rec["xcd"]),
+                         "xcd_busy_mean": sum(x["busy"] for x in rec["xcd"]) / len(rec["xcd"]),
+                         "tiles_per_workgroup_min": min(x["tiles_min"] for x in rec["xcd"]),
+                         "tiles_per_workgroup_max": max(x["tiles_max"] for x in rec["xcd"])}
+        return out
 
 
 def _other_configs(pkg, dev, headline, steps, warmup):
@@ -326,7 +346,15 @@ def main():
         "end_to_end": dict(s["end_to_end"], tops=work["ops"] / sec_per_pass / 1e12, gbps=work["bytes"] / sec_per_pass / 1e9),
         "kernels_ms": s["kernels_ms"],
         "roofline": s["roofline"],
+        "gemm_tile_balance": s["gemm_tile_balance"],
     }
+    # what the matrix pipe sustains with nothing else going on: the clock under matrix load follows the switching
+    # activity of the operands, so uniform random bytes (the benchmark's weights) run well below all-zero operands
+    result["int8_mfma_rate_probe"] = {
+        "zero_operands_tops": aclnn.int8_mfma_rate_probe(False) / 1e12,
+        "uniform_random_operands_tops": aclnn.int8_mfma_rate_probe(True) / 1e12,
+        "note": "back-to-back v_mfma_i32_32x32x32_i8 on register operands, 8 waves per CU, no memory traffic; "
+                "roofline.peak stays the published 5000 TOP/s"}
     if not args.no_cpu_baseline:
         oracle = graft.load_oracle()
         oracle.build()

@@ -36,6 +36,34 @@ __attribute__((visibility("default"))) int opapiKernelTimerReport(char* buf, siz
  */
 __attribute__((visibility("default"))) int opapiCalibrationCopy(void* dst, const void* src, size_t bytes, void* stream);
 
+/*
+ * Matrix-pipe rate probe: runs nothing but back-to-back v_mfma_i32_32x32x32_i8 on register operands (eight waves per CU,
+ * one workgroup per CU, `iterations` x 16 MFMAs per wave, one warm-up launch and one timed launch on the null stream)
+ * and writes the achieved int8 operations per second (2 per multiply-add).  uniformRandomOperands = 0: all-zero operands;
+ * non-zero: every operand byte uniform over [-127, 127], like the benchmark's weights.  The engine clock under matrix load
+ * follows the switching activity of the operands, so the second figure is the ceiling for a GEMM on such data.  Allocates
+ * and frees a few KB of device memory and synchronises: a measurement call, not for use inside a serving loop.
+ * Returns 0 or an aclnn status code.
+ */
+__attribute__((visibility("default"))) int opapiInt8MfmaRateProbe(int uniformRandomOperands, int iterations,
+                                                                  double* opsPerSecond);
+
+/*
+ * Workgroup spans of the grouped GEMM's persistent kernels: a measurement of how evenly the static deal of tiles to the
+ * workgroups (hence to the eight XCDs) ends.  While on, every workgroup of a ring-kernel launch records when it started
+ * and ended (the GPU's 100 MHz real-time counter) and how many tiles it computed; only the last launch of each kind
+ * (gmm_swiglu, gmm_dequant, gmm_int32) is kept.  Off by default; costs one branch per workgroup when off.
+ */
+__attribute__((visibility("default"))) void opapiGemmWorkgroupSpansEnable(int enable);
+
+/*
+ * Synchronises the device, then writes one text line per recorded kind into buf (NUL-terminated):
+ * "<name> workgroups <n> tile_rows <r> span_us <last end - first start>" followed, per XCD x = 0..7, by
+ * " xcd<x> end_us <when its last workgroup ended> busy <mean (end - start) / span of its workgroups> tiles <min>-<max>".
+ * Returns the number of lines, or -1 on an error.
+ */
+__attribute__((visibility("default"))) int opapiGemmWorkgroupSpansReport(char* buf, size_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -555,6 +555,48 @@ def kernel_timer_report():
     return out
 
 
+def gemm_workgroup_spans_enable(enable=True):
+    """Turns the recording of per-workgroup start / end times in the grouped GEMM's persistent kernels on or off."""
+    l = lib()
+    l.opapiGemmWorkgroupSpansEnable.argtypes = [ctypes.c_int]
+    l.opapiGemmWorkgroupSpansEnable.restype = None
+    l.opapiGemmWorkgroupSpansEnable(1 if enable else 0)
+
+
+def gemm_workgroup_spans_report():
+    """{kernel kind: {"workgroups", "tile_rows", "span_us", "xcd": [{"end_us", "busy", "tiles_min", "tiles_max"} x 8]}}
+    for the last launch of each kind (include/opapi_profile.h)."""
+    l = lib()
+    l.opapiGemmWorkgroupSpansReport.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
+    l.opapiGemmWorkgroupSpansReport.restype = ctypes.c_int
+    buf = ctypes.create_string_buffer(1 << 14)
+    if l.opapiGemmWorkgroupSpansReport(buf, len(buf)) < 0:
+        raise RuntimeError("opapiGemmWorkgroupSpansReport failed")
+    out = {}
+    for line in buf.value.decode().splitlines():
+        f = line.split()
+        rec = {"workgroups": int(f[2]), "tile_rows": int(f[4]), "span_us": float(f[6]), "xcd": []}
+        i = 7
+        while i < len(f):
+            tmin, tmax = f[i + 6].split("-")
+            rec["xcd"].append({"end_us": float(f[i + 2]), "busy": float(f[i + 4]), "tiles_min": int(tmin), "tiles_max": int(tmax)})
+            i += 7
+        out[f[0]] = rec
+    return out
+
+
+def int8_mfma_rate_probe(uniform_random_operands, iterations=20000):
+    """int8 operations per second of back-to-back MFMAs on register operands (include/opapi_profile.h)."""
+    l = lib()
+    l.opapiInt8MfmaRateProbe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    l.opapiInt8MfmaRateProbe.restype = ctypes.c_int
+    out = ctypes.c_double(0.0)
+    rc = l.opapiInt8MfmaRateProbe(1 if uniform_random_operands else 0, iterations, ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError("opapiInt8MfmaRateProbe failed with status %d" % rc)
+    return out.value
+
+
 def calibration_copy(dst, src):
     """Runs the library's plain copy kernel (include/opapi_profile.h) from src to dst, two same-sized device tensors."""
     assert dst.is_contiguous() and src.is_contiguous() and dst.numel() * dst.element_size() == src.numel() * src.element_size()

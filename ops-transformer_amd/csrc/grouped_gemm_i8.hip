@@ -213,6 +213,9 @@ struct KernelArgs {
     const float* combineWeight;
     const void* bias;
     int32_t biasDtype;
+    // workgroup spans (include/opapi_profile.h): per workgroup {start, end} of the 100 MHz real-time counter and the
+    // number of tiles it computed; null unless span recording is on
+    uint64_t* wgSpans;
 };
 
 // One output tile of one group, decoded from the scheduling table (all fields are wave-uniform).
@@ -638,9 +641,18 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     const int64_t slots = gridDim.x / kXcds;
     auto decode = [&](int64_t local) __attribute__((always_inline)) { return DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, local); };
 
+    const uint64_t spanStart = a.wgSpans != nullptr ? __builtin_amdgcn_s_memrealtime() : 0;
+    uint64_t spanTiles = 0;
     int64_t local = blockIdx.x / kXcds;
     TileInfo cur = decode(local);
-    if (!cur.valid) return;
+    if (!cur.valid) {
+        if (a.wgSpans != nullptr && tid == 0) {
+            a.wgSpans[3 * blockIdx.x] = spanStart;
+            a.wgSpans[3 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime();
+            a.wgSpans[3 * blockIdx.x + 2] = 0;
+        }
+        return;
+    }
     const int kSteps = a.K / kStep;
     // Small tiles are the decode shapes: a handful of rows per expert, every weight byte used once, pure streaming.
     constexpr bool kSmallTile = kTileM <= 64;
@@ -903,11 +915,17 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
         // stores and the DMAs in flight, which had the whole epilogue to land) before counting DMAs again.
         WaitVmcnt<0>();
+        ++spanTiles;
         if (!following.valid) break;
         __syncthreads();  // the epilogue's reads of ldsRowScale / ldsRowMax are done
         if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) ldsRowScale[tid] = followingRowScale;
         cur = following;
         local += slots;
+    }
+    if (a.wgSpans != nullptr && tid == 0) {
+        a.wgSpans[3 * blockIdx.x] = spanStart;
+        a.wgSpans[3 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime();
+        a.wgSpans[3 * blockIdx.x + 2] = spanTiles;
     }
 }
 
@@ -1083,6 +1101,25 @@ int DeviceCuCount() {
     return count;
 }
 
+// ---- workgroup spans (opapiGemmWorkgroupSpans*, include/opapi_profile.h): a measurement aid, off by default ----
+constexpr int kSpanKinds = 3;        // indexed by Epilogue
+constexpr int kSpanMaxGrid = 1024;
+std::atomic<int> gSpansOn{0};
+uint64_t* gSpanBuf[kSpanKinds] = {nullptr, nullptr, nullptr};
+int gSpanGrid[kSpanKinds] = {0, 0, 0};
+int gSpanTileM[kSpanKinds] = {0, 0, 0};
+
+// Device buffer for the next ring-kernel launch of this epilogue kind (allocated on first use, cleared on the stream),
+// or null when recording is off.
+uint64_t* SpanBufferFor(Epilogue epi, int grid, int tileM, hipStream_t stream) {
+    if (gSpansOn.load(std::memory_order_relaxed) == 0 || grid > kSpanMaxGrid) return nullptr;
+    const int k = static_cast<int>(epi);
+    if (gSpanBuf[k] == nullptr && hipMalloc(&gSpanBuf[k], kSpanMaxGrid * 3 * sizeof(uint64_t)) != hipSuccess) return nullptr;
+    gSpanGrid[k] = grid;
+    gSpanTileM[k] = tileM;
+    return gSpanBuf[k];
+}
+
 template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor>
 hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
     using Cfg = StreamCfg<kSub0, kSub1, kStep>;
@@ -1095,7 +1132,9 @@ hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t ma
     if (grid > maxTiles) grid = maxTiles;
     grid = grid / kXcds * kXcds;
     if (grid < kXcds) grid = kXcds;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, args, sched);
+    KernelArgs launchArgs = args;
+    launchArgs.wgSpans = SpanBufferFor(kEpi, static_cast<int>(grid), Cfg::kTileM, stream);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, launchArgs, sched);
     return hipGetLastError();
 }
 
@@ -1249,6 +1288,7 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.combineWeight = p.combineWeight;
     ka.bias = p.bias;
     ka.biasDtype = p.biasDtype;
+    ka.wgSpans = nullptr;
 
     hipError_t e = hipSuccess;
     if (p.K > 0) {
@@ -1282,3 +1322,57 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
 }
 
 }  // namespace gemm
+
+extern "C" __attribute__((visibility("default"))) void opapiGemmWorkgroupSpansEnable(int enable) {
+    gemm::gSpansOn.store(enable ? 1 : 0, std::memory_order_relaxed);
+}
+
+extern "C" __attribute__((visibility("default"))) int opapiGemmWorkgroupSpansReport(char* buf, size_t cap) {
+    using namespace gemm;
+    if (buf == nullptr || cap == 0) return -1;
+    if (hipDeviceSynchronize() != hipSuccess) return -1;
+    static const char* const kNames[kSpanKinds] = {"gmm_int32", "gmm_dequant", "gmm_swiglu"};
+    size_t used = 0;
+    int lines = 0;
+    buf[0] = 0;
+    std::vector<uint64_t> host(kSpanMaxGrid * 3);
+    for (int k = 0; k < kSpanKinds; ++k) {
+        const int grid = gSpanGrid[k];
+        if (gSpanBuf[k] == nullptr || grid <= 0) continue;
+        if (hipMemcpy(host.data(), gSpanBuf[k], static_cast<size_t>(grid) * 3 * sizeof(uint64_t), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+        uint64_t first = ~0ull, last = 0;
+        for (int b = 0; b < grid; ++b) {
+            first = std::min(first, host[3 * b]);
+            last = std::max(last, host[3 * b + 1]);
+        }
+        const double span = static_cast<double>(last - first) / 100.0;  // 100 MHz counter -> microseconds
+        int n = snprintf(buf + used, cap - used, "%s workgroups %d tile_rows %d span_us %.1f", kNames[k], grid, gSpanTileM[k], span);
+        if (n < 0 || static_cast<size_t>(n) >= cap - used) break;
+        used += static_cast<size_t>(n);
+        // per XCD (workgroup b runs on XCD b % 8): when its last workgroup ended, relative to the launch's first start,
+        // the mean busy fraction of its workgroups over the whole span, and the fewest / most tiles one of them took
+        for (int x = 0; x < kXcds; ++x) {
+            uint64_t xLast = 0, tMin = ~0ull, tMax = 0;
+            double busy = 0.0;
+            int count = 0;
+            for (int b = x; b < grid; b += kXcds) {
+                xLast = std::max(xLast, host[3 * b + 1]);
+                busy += static_cast<double>(host[3 * b + 1] - host[3 * b]);
+                tMin = std::min(tMin, host[3 * b + 2]);
+                tMax = std::max(tMax, host[3 * b + 2]);
+                ++count;
+            }
+            n = snprintf(buf + used, cap - used, " xcd%d end_us %.1f busy %.3f tiles %llu-%llu", x,
+                         static_cast<double>(xLast - first) / 100.0,
+                         span > 0 && count > 0 ? busy / 100.0 / count / span : 0.0, (unsigned long long)tMin, (unsigned long long)tMax);
+            if (n < 0 || static_cast<size_t>(n) >= cap - used) break;
+            used += static_cast<size_t>(n);
+        }
+        if (used + 2 < cap) {
+            buf[used++] = '\n';
+            buf[used] = 0;
+        }
+        ++lines;
+    }
+    return lines;
+}
