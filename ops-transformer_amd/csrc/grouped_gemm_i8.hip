@@ -522,10 +522,21 @@ __device__ __forceinline__ void ForCount(int count, F& f) {
 }
 
 // ---------------------------------------------------------------------------------------------- fast path: LDS-DMA ring
-// kStep = k-bytes per ring stage: 128 streams weights in whole 128-byte lines (best HBM efficiency) when three such
-// stages fit in LDS, 64 allows a deeper ring for the tall tiles.
+// kStep = k-bytes per ring stage: 128 streams weights in whole 128-byte lines (best HBM efficiency).
 // The tile's rows are split over one or two wave rows: wave row 0 owns kSub0 MFMA tiles (32 rows each), wave row 1 the
 // next kSub1 (kSub1 <= kSub0; kSub1 == 0 means four waves only).
+//
+// A stage is kTileM activation rows and kTileN weight channels of kStep k-bytes each.  Every wave fetches, per stage,
+// instructions wave, wave + kWaves, ... of the stage's list (activation part first, then weight part).
+//
+// Common depth (every height but 192 rows): a ring of whole stages.
+//
+// Staggered depths (192 rows).  Whole stages fit twice there, but three weight stages and two activation stages fit as
+// well -- and the depth matters for the weights, which come out of HBM, not for the activation rows, which the n-tiles
+// of an expert re-read from L2.  So the two parts live in rings of their own depth (the activation ring first), and
+// each has its own issue cursor: at k-step s a wave issues its activation share of step s + 2 and then its weight share
+// of step s + 3.  A wave's loads return in issue order; with the activation share going out first, "at most one weight
+// share outstanding" certifies both the activation stage issued one step ago and the weight stage issued two steps ago.
 template <int kSub0, int kSub1, int kStep>
 struct StreamCfg {
     static_assert(kSub1 <= kSub0, "wave row 0 is the taller one");
@@ -533,20 +544,31 @@ struct StreamCfg {
     static constexpr int kWaves = kWavesN * kWavesM;
     static constexpr int kThreads = 64 * kWaves;
     static constexpr int kTileM = 32 * (kSub0 + kSub1);
-    static constexpr int kStageBytes = (kTileM + kTileN) * kStep;
+    static constexpr int kStageBytesA = kTileM * kStep;
+    static constexpr int kStageBytesB = kTileN * kStep;
     static constexpr int kScratchBytes = (1 + kWavesN) * kTileM * 4;
-    static constexpr int kStagesFit = (kLdsBudget - kScratchBytes) / kStageBytes;
-    static constexpr int kStages = kStagesFit > 8 ? 8 : kStagesFit;
-    static constexpr int kLdsBytes = kStages * kStageBytes + kScratchBytes;
+    static constexpr bool kStaggered = kTileM == 192;
+    static constexpr int kFitWhole = (kLdsBudget - kScratchBytes) / (kStageBytesA + kStageBytesB);
+    static constexpr int kStagesB = kStaggered ? (kLdsBudget - kScratchBytes - 2 * kStageBytesA) / kStageBytesB
+                                               : (kFitWhole > 8 ? 8 : kFitWhole);
+    static constexpr int kStagesA = kStaggered ? 2 : kStagesB;
+    static constexpr int kLdsBytes = kStagesA * kStageBytesA + kStagesB * kStageBytesB + kScratchBytes;
     // one DMA instruction moves 64 lanes x 16 bytes = kRowsPerInstr tile rows of kStep k-bytes
     static constexpr int kChunksPerRow = kStep / kChunk;
     static constexpr int kRowsPerInstr = 64 / kChunksPerRow;
     static constexpr int kInstrA = kTileM / kRowsPerInstr;
-    static constexpr int kInstr = (kTileM + kTileN) / kRowsPerInstr;
+    static constexpr int kInstrB = kTileN / kRowsPerInstr;
+    static constexpr int kInstr = kInstrA + kInstrB;
     static_assert(kTileM % kRowsPerInstr == 0, "tile rows must fill whole DMA instructions");
+    // Every wave issues exactly kMaxPerWave DMA instructions per stage: slots past the last instruction repeat it (same
+    // bytes to the same place), which keeps the issue code free of branches and the vmcnt arithmetic uniform.
     static constexpr int kMaxPerWave = (kInstr + kWaves - 1) / kWaves;
-    static_assert(kStages >= 2, "the ring needs at least two stages");
-    static_assert((kStages - 1) * kMaxPerWave <= 63, "vmcnt is a 6-bit counter");
+    // staggered depths: the first kSlotsA slots of every wave are activation instructions, the others weight instructions
+    static constexpr int kSlotsA = kInstrA / kWaves;
+    static constexpr int kSlotsB = kMaxPerWave - kSlotsA;
+    static_assert(!kStaggered || (kInstrA % kWaves == 0 && kInstrB % kWaves == 0), "the same split of slots in every wave");
+    static_assert(kStagesA >= 2 && kStagesB >= kStagesA, "each ring needs at least two stages");
+    static_assert(kStagesB * kMaxPerWave <= 63, "vmcnt is a 6-bit counter");
 };
 
 // Byte offset of 16-byte chunk `chunk` of row `row` in a stage whose rows are kStep bytes.  The LDS serves 16 lanes per
@@ -592,6 +614,15 @@ __device__ __forceinline__ void DmaToLdsAddr16(const char* base, uint32_t laneOf
     }
 }
 
+// The value itself, through a statement the optimiser cannot see through: what is computed from the copy stays where it
+// is written.  Used on lane indices at the head of per-tile code, so that the per-lane offsets and addresses of that code
+// are recomputed once per tile instead of being hoisted out of the tile loop and held in registers (or spilled) across the
+// k loop, where the accumulators and fragments of the tallest tiles leave no room for them.
+__device__ __forceinline__ int Opaque(int v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 template <int kCount>
 __device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leaving expcnt / lgkmcnt untouched
     __builtin_amdgcn_s_waitcnt(0x0f70 | (kCount & 15) | ((kCount >> 4) << 14));
@@ -620,11 +651,17 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     using Cfg = StreamCfg<kSub0, kSub1, kStep>;
     constexpr int kSubM = kSub0;  // accumulator tiles per wave (wave row 1 uses the first kSub1 of them)
     constexpr int kTileM = Cfg::kTileM;
-    constexpr int kStages = Cfg::kStages;
-    constexpr int kStageBytes = Cfg::kStageBytes;
+    constexpr int kStagesA = Cfg::kStagesA, kStagesB = Cfg::kStagesB;
+    constexpr int kStageBytesA = Cfg::kStageBytesA, kStageBytesB = Cfg::kStageBytesB;
+    // LDS layout.  Common depth: stage after stage, each its activation part followed by its weight part.  Staggered
+    // depths: the ring of activation stages, behind it the ring of weight stages.
+    constexpr bool kStaggered = Cfg::kStaggered;
+    constexpr int kStrideA = kStaggered ? kStageBytesA : kStageBytesA + kStageBytesB;  // from one activation stage to the next
+    constexpr int kStrideB = kStaggered ? kStageBytesB : kStageBytesA + kStageBytesB;
+    constexpr int kFirstB = kStaggered ? kStagesA * kStageBytesA : kStageBytesA;       // weight part of stage 0
     constexpr bool kSwiglu = kEpi == Epilogue::kSwiglu;
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    float* const ldsRowScale = reinterpret_cast<float*>(lds + kStages * kStageBytes);  // [kTileM]
+    float* const ldsRowScale = reinterpret_cast<float*>(lds + kStagesA * kStageBytesA + kStagesB * kStageBytesB);  // [kTileM]
     float* const ldsRowMax = ldsRowScale + kTileM;                                      // [kWavesN][kTileM]
 
     const int tid = threadIdx.x;
@@ -658,130 +695,195 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     constexpr bool kSmallTile = kTileM <= 64;
     const int kRotate = kSmallTile ? static_cast<int>((blockIdx.x * 7u + blockIdx.x / kXcds) % static_cast<unsigned>(kSteps)) : 0;
 
-    // ---- issue side: runs kStages - 1 steps ahead of the compute side, across tile boundaries ----
+    // ---- issue side: runs ahead of the compute side by the depth of the ring(s), across tile boundaries ----
+    // A cursor walks this workgroup's tiles k-step by k-step.  Cursor B drives the weight part -- and the activation
+    // part too where the depths are the same; with staggered depths the activation part has cursor A, one k-step behind.
+    // (Plain variables, picked by if constexpr: a cursor struct handed round by reference ends up in vector registers.)
     const uint32_t ldsBase = LdsAddress(lds);
-    TileInfo iss = cur;
-    int64_t issLocal = local;
-    int issStep = 0;
-    bool issDrained = false;  // no further tile: the remaining issue slots re-read one hot kilobyte (see below)
-    const char* issX = nullptr;
-    const char* issW = nullptr;
+    TileInfo issTileA = cur, issTileB = cur;
+    int64_t issLocalA = local, issLocalB = local;
+    int issStepA = 0, issStepB = 0;            // k-step of the tile that goes out next
+    int issSlotA = 0, issSlotB = 0;            // ring buffer it goes into
+    bool issDrainedA = false, issDrainedB = false;  // no further tile: the issue slots re-read one hot kilobyte (see advance)
+    const char* issBaseA = nullptr;  // the tile's activation rows
+    const char* issBaseB = nullptr;  // its expert's weights
     uint32_t laneOff[Cfg::kMaxPerWave];
-    // Every wave issues exactly kMaxPerWave DMA instructions per stage: slots past the last instruction repeat it (same
-    // bytes to the same place), which keeps the issue code free of branches and the vmcnt arithmetic uniform.
+    constexpr int kPartA = 1, kPartB = 2, kBothParts = 3;
+    using PartATag = std::integral_constant<int, kPartA>;
+    using PartBTag = std::integral_constant<int, kPartB>;
+    using BothPartsTag = std::integral_constant<int, kBothParts>;
+    // instruction of slot q in the stage's list (activation part, then weight part)
+    auto slotInstr = [&](int q) __attribute__((always_inline)) { return min(wave + q * Cfg::kWaves, Cfg::kInstr - 1); };
 
     // The lambdas below are forced inline: left to the inliner's size heuristics, one of them staying a real call puts
     // the whole issue state (captured by reference) into scratch memory and the kernel runs three times slower.
-    auto setupIssue = [&]() __attribute__((always_inline)) {
-        issX = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(iss.rowBase) * a.K;
-        issW = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(iss.group) * a.wGroupStride;
+    // Bases and lane offsets of the given part(s) for tile t.
+    auto setupIssue = [&](const TileInfo& t, auto partsTag) __attribute__((always_inline)) {
+        constexpr int kParts = decltype(partsTag)::value;
+        if (kParts & kPartA) issBaseA = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(t.rowBase) * a.K;
+        if (kParts & kPartB) issBaseB = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(t.group) * a.wGroupStride;
         // lane -> (row inside the instruction, LDS chunk slot); the global chunk it fetches is the one LdsOffset puts there
+        const int lane = Opaque(tid & 63);
         const int rowIn = lane / Cfg::kChunksPerRow;
         const int slot = lane % Cfg::kChunksPerRow;
 #pragma unroll
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
-            const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
-            if (j < Cfg::kInstrA) {
+            if (kParts != kBothParts && (q < Cfg::kSlotsA) != (kParts == kPartA)) continue;
+            const int g = slotInstr(q);
+            const int j = g < Cfg::kInstrA ? g : g - Cfg::kInstrA;  // instruction of its part
+            if (g < Cfg::kInstrA) {
                 // rows past the tile's last row are never used: such lanes re-read the last real row (same cache
                 // lines as its own lanes), and an instruction wholly past it reads one chunk, so the number of DMAs
                 // per stage stays constant while the activation traffic follows the real row count
                 const int r = Cfg::kRowsPerInstr * j + rowIn;
                 const int c = (LdsOffset<kStep>(r, slot) >> 4) % Cfg::kChunksPerRow;
-                const bool wholeInstrPast = Cfg::kRowsPerInstr * j >= iss.rows;
-                laneOff[q] = wholeInstrPast ? 0u : static_cast<uint32_t>(min(r, iss.rows - 1) * a.K + c * kChunk);
+                const bool wholeInstrPast = Cfg::kRowsPerInstr * j >= t.rows;
+                laneOff[q] = wholeInstrPast ? 0u : static_cast<uint32_t>(min(r, t.rows - 1) * a.K + c * kChunk);
             } else if (kNMajor) {
-                // weight instruction jw moves k-rows 4 * jw .. + 3 of the stage, 256 channel bytes each; lane ->
+                // weight instruction j moves k-rows 4 * j .. + 3 of the stage, 256 channel bytes each; lane ->
                 // (k-row lane / 16, LDS chunk slot lane % 16), fetching the logical chunk that the swizzle puts there.
                 // Chunks past the last channel are never stored: such lanes re-read the last real chunk.
-                const int jw = j - Cfg::kInstrA;
-                const int k = 4 * jw + lane / 16;
+                const int k = 4 * j + lane / 16;
                 const int c = (lane % 16) ^ ((k & 7) << 1);
                 int32_t col;
                 if (kSwiglu) {
-                    col = c < 8 ? min(iss.colBase + 16 * c, a.halfN - 16) : min(a.halfN + iss.colBase + 16 * (c - 8), a.N - 16);
+                    col = c < 8 ? min(t.colBase + 16 * c, a.halfN - 16) : min(a.halfN + t.colBase + 16 * (c - 8), a.N - 16);
                 } else {
-                    col = min(iss.colBase + 16 * c, a.N - 16);
+                    col = min(t.colBase + 16 * c, a.N - 16);
                 }
                 laneOff[q] = static_cast<uint32_t>(k * a.N + col);
             } else if (kNz) {
-                // weight instruction jw moves 32 k-rows (x 32 channel bytes) of channel block jw / 4: 1 KB, contiguous
+                // weight instruction j moves 32 k-rows (x 32 channel bytes) of channel block j / 4: 1 KB, contiguous
                 // in memory and in LDS; lane -> (k-row lane / 2, 16-byte half lane % 2)
-                const int jw = j - Cfg::kInstrA;
-                const int32_t block = ChannelOfRow<kSwiglu>(a, iss, 32 * (jw / 4)) >> 5;
-                laneOff[q] = static_cast<uint32_t>(block * a.K * 32 + ((jw % 4) * 32 + lane / 2) * 32 + (lane % 2) * kChunk);
+                const int32_t block = ChannelOfRow<kSwiglu>(a, t, 32 * (j / 4)) >> 5;
+                laneOff[q] = static_cast<uint32_t>(block * a.K * 32 + ((j % 4) * 32 + lane / 2) * 32 + (lane % 2) * kChunk);
             } else {
-                const int r = Cfg::kRowsPerInstr * (j - Cfg::kInstrA) + rowIn;
+                const int r = Cfg::kRowsPerInstr * j + rowIn;
                 const int c = (LdsOffset<kStep>(r, slot) >> 4) % Cfg::kChunksPerRow;
-                laneOff[q] = static_cast<uint32_t>(ChannelOfRow<kSwiglu>(a, iss, r) * a.K + c * kChunk);
+                laneOff[q] = static_cast<uint32_t>(ChannelOfRow<kSwiglu>(a, t, r) * a.K + c * kChunk);
             }
         }
     };
-    // DMA instruction q (0 .. kMaxPerWave - 1) of this wave's share of the stage at the issue cursor, into buffer `ring`.
-    auto issueOne = [&](int ring, int q) __attribute__((always_inline)) {
-        const uint32_t dst = ldsBase + ring * kStageBytes;
+    // Moves the cursor of the given part(s) to the next k-step (after the last instruction of a stage has gone out).
+    auto advance = [&](auto partsTag) __attribute__((always_inline)) {
+        constexpr int kParts = decltype(partsTag)::value;
+        constexpr bool kCursorA = kParts == kPartA;
+        TileInfo& tile = kCursorA ? issTileA : issTileB;
+        int64_t& tileLocal = kCursorA ? issLocalA : issLocalB;
+        int& step = kCursorA ? issStepA : issStepB;
+        int& slot = kCursorA ? issSlotA : issSlotB;
+        bool& drained = kCursorA ? issDrainedA : issDrainedB;
+        constexpr int kDepth = kCursorA ? kStagesA : kStagesB;
+        slot = slot + 1 == kDepth ? 0 : slot + 1;
+        if (++step == kSteps) {
+            // move to this workgroup's next tile.  Past the last one the issue slots still go out (that keeps the number
+            // of outstanding DMAs per stage, hence the vmcnt arithmetic, constant) into ring slots nobody reads -- but
+            // every one of them then re-reads the same first kilobyte of the last tile's weights, which stays in L2,
+            // instead of pulling more stages of weights from HBM per workgroup.
+            step = 0;
+            const TileInfo next = decode(tileLocal + slots);
+            if (next.valid) {
+                tile = next;
+                tileLocal += slots;
+                setupIssue(tile, partsTag);
+            } else if (!drained) {
+                drained = true;
+                // any mapped, 16-byte aligned kilobyte will do: the start of the last tile's expert's weights
+                const char* const hot = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(tile.group) * a.wGroupStride;
+                if (kParts & kPartA) issBaseA = hot;
+                if (kParts & kPartB) issBaseB = hot;
+#pragma unroll
+                for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
+                    if (kParts != kBothParts && (q < Cfg::kSlotsA) != (kParts == kPartA)) continue;
+                    laneOff[q] = static_cast<uint32_t>(lane) * kChunk;
+                }
+            }
+        }
+    };
+    // This wave's DMA instructions of the given part(s) of the stage at the part's cursor.
+    auto emitParts = [&](auto partsTag) __attribute__((always_inline)) {
+        constexpr int kParts = decltype(partsTag)::value;
+        constexpr bool kOwnA = kParts == kPartA;  // else the activation part, if any, follows cursor B
         // On small tiles the k-steps of a tile are walked from a start that differs between workgroups (integer
         // accumulation does not care about the order).  When rows lie a power-of-two stride apart (K = 4096 with
         // K-contiguous weights), the low address bits of every row of every expert depend on the k offset alone:
         // workgroups that all sit at the same k-step all queue on the same memory channels.  Only for small tiles, where
         // every weight byte is used once: on the large-tile shapes neighbouring workgroups share operands through L2,
         // and walking k in step is what makes those hits.
-        const int kIdx = issStep + kRotate;
-        const int kOff = issDrained ? 0 : (kIdx >= kSteps ? kIdx - kSteps : kIdx) * kStep;
-        // blocked layout: one k is 32 bytes further; row-major: N bytes
-        const int kOffW = kNz ? kOff * 32 : (kNMajor ? kOff * a.N : kOff);
-        const int j = min(wave + q * Cfg::kWaves, Cfg::kInstr - 1);
-        // wave-uniform branch: activation rows always stay cacheable (the n-tiles of a group re-read them from L2);
-        // on small tiles (every weight byte is used exactly once) the weights stream past the caches.  On large
-        // tiles the m-tiles of a group share their weight columns through L2 and must not.
-        if constexpr (kSmallTile) {
-            if (j < Cfg::kInstrA) DmaToLdsAddr16<false>(issX + kOff, laneOff[q], dst + j * 1024);
-            else DmaToLdsAddr16<true>(issW + kOffW, laneOff[q], dst + j * 1024);
-        } else {
-            DmaToLdsAddr16<false>(j < Cfg::kInstrA ? issX + kOff : issW + kOffW, laneOff[q], dst + j * 1024);
-        }
-    };
-    // Moves the issue cursor to the next k-step (after the last instruction of a stage has gone out).
-    auto issueAdvance = [&]() __attribute__((always_inline)) {
-        if (++issStep == kSteps) {
-            // move to this workgroup's next tile.  Past the last one the issue slots still go out (that keeps the number
-            // of outstanding DMAs per stage, hence the vmcnt arithmetic, constant) into ring slots nobody reads -- but
-            // every one of them then re-reads the same first kilobyte of the last tile's weights, which stays in L2,
-            // instead of pulling (stages - 1) more stages of weights from HBM per workgroup.
-            issStep = 0;
-            const TileInfo next = decode(issLocal + slots);
-            if (next.valid) {
-                iss = next;
-                issLocal += slots;
-                setupIssue();
-            } else if (!issDrained) {
-                issDrained = true;
-                issX = issW;  // any mapped, 16-byte aligned kilobyte will do
+        auto kOffset = [&](int step, bool drained) __attribute__((always_inline)) {
+            const int kIdx = step + kRotate;
+            return drained ? 0 : (kIdx >= kSteps ? kIdx - kSteps : kIdx) * kStep;
+        };
+        const int kOffB = kOffset(issStepB, issDrainedB);
+        const int kOffA = kOwnA ? kOffset(issStepA, issDrainedA) : kOffB;
+        // weights -- blocked layout: one k is 32 bytes further; row-major: N bytes
+        const int kOffW = kNz ? kOffB * 32 : (kNMajor ? kOffB * a.N : kOffB);
+        // instruction g lands g KB behind dstA (activation part) or dstB (weight part, whose first instruction is kInstrA)
+        const uint32_t dstA = ldsBase + (kOwnA ? issSlotA : issSlotB) * kStrideA;
+        const uint32_t dstB = ldsBase + kFirstB + issSlotB * kStrideB - Cfg::kInstrA * 1024;
 #pragma unroll
-                for (int q = 0; q < Cfg::kMaxPerWave; ++q) laneOff[q] = static_cast<uint32_t>(lane) * kChunk;
+        for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
+            if (kParts != kBothParts && (q < Cfg::kSlotsA) != (kParts == kPartA)) continue;
+            const int g = slotInstr(q);
+            const bool isA = g < Cfg::kInstrA;
+            // wave-uniform choice: activation rows always stay cacheable (the n-tiles of a group re-read them from L2);
+            // on small tiles (every weight byte is used exactly once) the weights stream past the caches.  On large
+            // tiles the m-tiles of a group share their weight columns through L2 and must not.
+            if constexpr (kSmallTile) {
+                if (isA) DmaToLdsAddr16<false>(issBaseA + kOffA, laneOff[q], dstA + g * 1024);
+                else DmaToLdsAddr16<true>(issBaseB + kOffW, laneOff[q], dstB + g * 1024);
+            } else {  // selects, no branch: the k-step stays one basic block
+                DmaToLdsAddr16<false>(isA ? issBaseA + kOffA : issBaseB + kOffW, laneOff[q], (isA ? dstA : dstB) + g * 1024);
             }
         }
     };
-
-    // A whole stage at once: every instruction of this wave's share, then the cursor moves on.
-    auto issueStage = [&](int ring) __attribute__((always_inline)) {
-#pragma unroll
-        for (int q = 0; q < Cfg::kMaxPerWave; ++q) issueOne(ring, q);
-        issueAdvance();
+    // One k-step's worth of issue: a whole stage, or (staggered depths) the activation share and then the weight share,
+    // each of the stage its own cursor has reached.
+    // The cursors move when all of it has gone out, so that the DMAs of a k-step stay in one basic block.
+    auto issueStage = [&]() __attribute__((always_inline)) {
+        if constexpr (kStaggered) {
+            emitParts(PartATag{});
+            emitParts(PartBTag{});
+            advance(PartATag{});
+            advance(PartBTag{});
+        } else {
+            emitParts(BothPartsTag{});
+            advance(BothPartsTag{});
+        }
+    };
+    // vmcnt that certifies the stage the compute side needs next with `younger` whole k-steps' worth of issue behind it
+    // (staggered depths: and that stage's own weight share, which went out after its activation share)
+    auto waitStage = [&](auto tag) __attribute__((always_inline)) {
+        constexpr int kYounger = decltype(tag)::value;
+        WaitVmcnt<kYounger * Cfg::kMaxPerWave + (kStaggered ? Cfg::kSlotsB : 0)>();
     };
 
     // Shifted barrier (tall tiles).  The plain k-step opens with its barrier -- the stage has landed, the previous one is
     // no longer read -- after which every wave waits for its first fragments before it has any MFMA to issue.  Here the
     // step's one barrier sits in front of its LAST block of MFMAs instead: by then every k-slice of the stage has been
-    // read, so the buffer takes its refill a quarter of a step earlier, the same barrier certifies the next stage as
+    // read, so the buffers take their refill a quarter of a step earlier, the same barrier certifies the next stage as
     // landed, and the next step's first fragments are read while the matrix pipe still has a block of MFMAs to run.  All
-    // kStages buffers are in use.
+    // buffers of both rings are in use.
     constexpr bool kEarly = kTileM >= 96;
-    setupIssue();
+    static_assert(!kStaggered || kEarly, "staggered depths are built on the shifted barrier");
+    setupIssue(cur, BothPartsTag{});
+    if constexpr (kStaggered) {
+        // the order the steady state would have left behind: weight stages 0 .. kStagesB - kStagesA - 1 alone, then
+        // (activation stage i, weight stage kStagesB - kStagesA + i) for i = 0 .. kStagesA - 1
 #pragma unroll 1
-    for (int s = 0; s < (kEarly ? kStages : kStages - 1); ++s) issueStage(s);
-    int ring = 0;  // stage the compute side reads next; the issue side writes (ring + kStages - 1) % kStages (kEarly: ring itself)
+        for (int s = 0; s < kStagesB - kStagesA; ++s) {
+            emitParts(PartBTag{});
+            advance(PartBTag{});
+        }
+#pragma unroll 1
+        for (int s = 0; s < kStagesA; ++s) issueStage();
+    } else {
+#pragma unroll 1
+        for (int s = 0; s < (kEarly ? kStagesB : kStagesB - 1); ++s) issueStage();
+    }
+    int ringA = 0, ringB = 0;  // buffers the compute side reads next (one index where the depths are the same)
     if constexpr (kEarly) {
-        WaitVmcnt<(kStages - 1) * Cfg::kMaxPerWave>();
+        waitStage(std::integral_constant<int, kStagesA - 1>{});
         __syncthreads();  // stage 0 has landed for every wave
     }
 
@@ -824,17 +926,17 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             static_assert(kSlices % 2 == 0, "the fragment double buffer is handed over between steps at slot 0");
             v4i bf[2][2];
             v4i af[2][kMy > 0 ? kMy : 1];
-            auto loadSlice = [&](int stage, int ks, int buf) __attribute__((always_inline)) {
+            auto loadSlice = [&](int stageA, int stageB, int ks, int buf) __attribute__((always_inline)) {
                 if (kMy == 0) return;
-                const char* const A = lds + stage * kStageBytes;
-                const char* const B = A + kTileM * kStep;
+                const char* const A = lds + (kStaggered ? stageA : stageB) * kStrideA;  // common depth: one ring index
+                const char* const B = lds + kFirstB + stageB * kStrideB;
                 const int chunk = 2 * ks + lhi;
                 if constexpr (kNMajor) {
                     // 16-lane group g: channels 16 * (g % 2) .. + 15 of the 32-channel block, k-half g / 2 (= lhi) of the
                     // slice; lane j of the group supplies bytes (k = kBase + j / 2, channels 8 * (j % 2) .. + 7)
                     const int j = lane & 15;
                     const int k = 32 * ks + 16 * lhi + (j >> 1);
-                    const uint32_t bBase = ldsBase + stage * kStageBytes + kTileM * kStep + 8 * (j & 1);
+                    const uint32_t bBase = ldsBase + kFirstB + stageB * kStrideB + 8 * (j & 1);
 #pragma unroll
                     for (int ni = 0; ni < 2; ++ni) {
                         const int c = (bRow0 + ni * bRowStep + 16 * ((lane >> 4) & 1)) >> 4;  // logical 16-byte chunk of the row
@@ -853,7 +955,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
 #pragma unroll
                     for (int ni = 0; ni < 2; ++ni) {
                         // addressed through the 32-bit LDS address: no generic-to-LDS pointer conversion in the loop
-                        const uint32_t blk = ldsBase + stage * kStageBytes + kTileM * kStep +
+                        const uint32_t blk = ldsBase + kFirstB + stageB * kStrideB +
                                              ((bRow0 + ni * bRowStep) >> 5) * 4096 + inBlock;
                         const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk));
                         const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk + 8 * 32));
@@ -868,39 +970,54 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                     af[buf][mi] = *reinterpret_cast<const v4i*>(A + LdsOffset<kStep>(waveRow0 + mi * 32 + l32, chunk));
                 }
             };
-            if constexpr (kEarly) loadSlice(ring, 0, 0);  // the tile's first stage was certified at the end of the tile before
+            if constexpr (kEarly) loadSlice(ringA, ringB, 0, 0);  // the tile's first stage was certified at the end of the tile before
 #pragma unroll 1
             for (int step = 0; step < kSteps; ++step) {
                 if constexpr (!kEarly) {
-                    // the oldest stage in flight has landed once at most (kStages - 2) stages' worth of this wave's DMAs remain
-                    WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
-                    __syncthreads();  // every wave's share of stage `ring` is in LDS, and stage ring - 1 is no longer read
-                    loadSlice(ring, 0, 0);
+                    // the oldest stage in flight has landed once at most (stages - 2) stages' worth of this wave's DMAs remain
+                    waitStage(std::integral_constant<int, kStagesA - 2>{});
+                    __syncthreads();  // every wave's share of the stage is in LDS, and the previous stage is no longer read
+                    loadSlice(ringA, ringB, 0, 0);
                 }
-                const int nextRing = ring + 1 == kStages ? 0 : ring + 1;
+                const int nextA = !kStaggered ? 0 : ringA + 1 == kStagesA ? 0 : ringA + 1;  // unused with a common depth
+                const int nextB = ringB + 1 == kStagesB ? 0 : ringB + 1;
 #pragma unroll
                 for (int ks = 0; ks < kSlices; ++ks) {
                     if (!kEarly || ks + 1 < kSlices) {
-                        if (ks + 1 < kSlices) loadSlice(ring, ks + 1, (ks + 1) & 1);
+                        if (ks + 1 < kSlices) loadSlice(ringA, ringB, ks + 1, (ks + 1) & 1);
                     } else {
                         // Before the step's last block of MFMAs: every k-slice of this stage has been read (the reads
                         // of the last one returned in the shadow of the block before), and the next stage, issued one
                         // step ago, should have landed.  One barrier certifies both; inside a tile, the next step's
                         // first fragments are read behind the MFMAs.
                         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads have returned
-                        WaitVmcnt<(kStages - 2) * Cfg::kMaxPerWave>();
+                        waitStage(std::integral_constant<int, kStagesA - 2>{});
                         __syncthreads();
-                        issueStage(ring);
-                        if (step + 1 < kSteps) loadSlice(nextRing, 0, 0);
+                        issueStage();  // into the buffer(s) that this step read
+                        if (step + 1 < kSteps) loadSlice(nextA, nextB, 0, 0);
                     }
 #pragma unroll
                     for (int mi = 0; mi < kMy; ++mi) {
                         acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][0], acc[mi][0], 0, 0, 0);
                         acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][1], acc[mi][1], 0, 0, 0);
                     }
-                    if (!kEarly && ks == 0) issueStage(ring == 0 ? kStages - 1 : ring - 1);
+                    if constexpr (kEarly && kMy > 0) {
+                        if (ks + 1 < kSlices) {
+                            // The k-slice's pipeline, pinned: the reads of the next slice go out behind the first MFMA
+                            // and return under the others.  Left alone, the scheduler makes this order on some builds
+                            // and, at the register limit of the tallest tiles, on others a late-read order that stalls
+                            // the matrix pipe.  (Reading each fragment only when the one before it has retired saves
+                            // registers and measures slower.)
+                            constexpr int kReads = kMy + ((kNz || kNMajor) ? 4 : 2);
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);       // the LDS reads
+                            __builtin_amdgcn_sched_group_barrier(0x008, 2 * kMy - 1, 0);  // the other MFMAs
+                        }
+                    }
+                    if (!kEarly && ks == 0) issueStage();  // into the buffer that the step before read
                 }
-                ring = nextRing;
+                ringA = nextA;
+                ringB = nextB;
             }
         };
         {
@@ -911,7 +1028,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         }
         ForCount<kSub0>(mySub, runTile);
 
-        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, waveN, l32, lhi, tid, ldsRowScale, ldsRowMax);
+        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, waveN, Opaque(l32), Opaque(lhi), Opaque(tid), ldsRowScale, ldsRowMax);
         // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
         // stores and the DMAs in flight, which had the whole epilogue to land) before counting DMAs again.
         WaitVmcnt<0>();
@@ -1138,8 +1255,8 @@ hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t ma
     return hipGetLastError();
 }
 
-// Tile heights and their (wave row 0, wave row 1, k-step) shapes.  128-byte steps with a ring of three or more stages
-// stream best; 192 and 256 rows only leave room for two such stages.
+// Tile heights and their (wave row 0, wave row 1, k-step) shapes.  Up to 192 rows the weight ring holds three or more
+// 128-byte stages; from 192 rows on the activation ring holds two.
 template <Epilogue kEpi, bool kNz, bool kNMajor>
 hipError_t LaunchStreamShapeOf(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
     switch (plan.tileM) {
@@ -1193,11 +1310,18 @@ uint64_t Align256(uint64_t v) { return (v + 255) / 256 * 256; }
 Plan MakePlan(const Problem& p) {
     Plan plan;
     const int64_t groups = p.groups > 0 ? p.groups : 1;
+    const int64_t cols = p.epilogue == Epilogue::kSwiglu ? p.N / 2 : p.N;
+    const int64_t colsPerTile = p.epilogue == Epilogue::kSwiglu ? kTileN / 2 : kTileN;
+    plan.tilesN = static_cast<int32_t>((cols + colsPerTile - 1) / colsPerTile);
     // tile height: the mean group size plus a quarter, so that almost every group is covered by one m-tile and its
-    // weights are streamed exactly once
+    // weights are streamed exactly once.  A group that still overflows its tile adds a second m-tile, i.e. tilesN more
+    // tiles, all in one XCD's share: its workgroups walk one round more than the others.  Where a workgroup walks few
+    // rounds (one is more than 4 % of the launch) the headroom is half the mean instead: the taller shapes pay for
+    // their extra rows with a shallower activation ring, which costs less than that round.
     const double meanRows = p.expectedRowsPerGroup > 0 ? static_cast<double>(p.expectedRowsPerGroup)
                                                        : static_cast<double>(p.M) / static_cast<double>(groups);
-    const double want = meanRows * 1.25;
+    const double rounds = static_cast<double>(groups) * plan.tilesN / DeviceCuCount();
+    const double want = meanRows * (rounds <= 24.0 ? 1.5 : 1.25);
     if (StreamOk(p)) {
         static const int kShapes[] = {32, 64, 96, 128, 160, 192, 256};
         plan.tileM = 256;
@@ -1216,9 +1340,6 @@ Plan MakePlan(const Problem& p) {
     }
     plan.wavesM = plan.tileM >= 64 && StreamOk(p) ? 2 : 1;
     plan.subTilesM = (plan.tileM / 32 + plan.wavesM - 1) / plan.wavesM;
-    const int64_t cols = p.epilogue == Epilogue::kSwiglu ? p.N / 2 : p.N;
-    const int64_t colsPerTile = p.epilogue == Epilogue::kSwiglu ? kTileN / 2 : kTileN;
-    plan.tilesN = static_cast<int32_t>((cols + colsPerTile - 1) / colsPerTile);
     const int64_t maxMTiles = p.M / plan.tileM + groups;
     plan.maxMTiles = static_cast<int32_t>(maxMTiles);
     // round up so that every XCD's share [xcd * ceil(total/8), ...) is covered by the launch
