@@ -17,9 +17,10 @@
 //
 // Two kernels share the tile decode and the epilogue:
 //   StreamGemmKernel  the fast path (K a multiple of 128; K-contiguous, blocked or row-major [K, N] weights).  Persistent workgroups; operands go
-//                     global -> LDS with global_load_lds_dwordx4 into a ring of 3..8 stages of 128 (or 64) k-bytes, so several
-//                     stages of weights are in flight per CU with no staging registers, and the ring keeps filling
-//                     with the next tile's first steps while the current tile's epilogue runs.
+//                     global -> LDS with global_load_lds_dwordx4 into a ring of 2..4 stages of 128 k-bytes (192-row tiles:
+//                     two activation and three weight stages), so several stages of weights are in flight per CU
+//                     with no staging registers, and the ring already holds the next tile's first steps while the
+//                     current tile's epilogue runs.
 //   GenericGemmKernel byte-wise loader for K not a multiple of 128 and channel counts off the 16-byte grid: correct, slow.
 // LDS rows are XOR-swizzled in 16-byte chunks so that the 16 lanes the LDS serves per clock (64 banks) never collide,
 // for the DMA writes as well as for the MFMA operand reads.

@@ -358,3 +358,54 @@ def test_every_tile_height_and_layout(aclnn, oracle, dev, monkeypatch, tile_m, l
     diff = np.abs(q.cpu().numpy().astype(np.int32) - q_ref.astype(np.int32))
     assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
     np.testing.assert_allclose(qs.cpu().numpy(), qs_ref, rtol=1e-5)
+
+
+@pytest.mark.parametrize("K", [128, 256, 640])
+@pytest.mark.parametrize("tile_m", [32, 64, 96, 128, 160, 192, 256])
+def test_many_tiles_per_workgroup_every_height(aclnn, oracle, dev, monkeypatch, tile_m, K):
+    """Every workgroup of the persistent kernel walks several tiles here, and a tile is one, two or five k-steps long --
+    shorter than the LDS ring is deep -- so the issue cursors run a tile or more ahead of the MFMAs, cross tile
+    boundaries at different times (the 192-row kernel keeps one cursor per operand) and drain at the end of the walk.
+    The forced-height test above has fewer tiles than workgroups and never gets there.  int32 output, bit-exact."""
+    monkeypatch.setenv("OPAPI_GEMM_TILE_M", str(tile_m))
+    rng = np.random.default_rng(1000 * tile_m + K)
+    E, N = 48, 256 * 8 + 64
+    sizes = rng.integers(0, 230, E)
+    sizes[5] = 0
+    sizes[17] = 257                      # one group past the tallest tile
+    cumsum = np.cumsum(sizes).astype(np.int64)
+    M = int(cumsum[-1])
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    acc = aclnn.grouped_matmul_v4([t(x)], [_weight_views(wt, dev, "kmajor")], group_list=t(cumsum), split_item=3, group_type=0)[0]
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True))
+
+
+@pytest.mark.parametrize("layout", ["nz", "nd"])
+@pytest.mark.parametrize("tile_m", [128, 192, 256])
+def test_many_tiles_per_workgroup_other_layouts(aclnn, oracle, dev, monkeypatch, tile_m, layout):
+    """The same walk with the blocked and the row-major weight layouts (bf16 output of the down projection as well)."""
+    monkeypatch.setenv("OPAPI_GEMM_TILE_M", str(tile_m))
+    rng = np.random.default_rng(31 * tile_m + len(layout))
+    E, N, K = 40, 256 * 8 + 64, 256
+    sizes = rng.integers(0, 230, E)
+    cumsum = np.cumsum(sizes).astype(np.int64)
+    M = int(cumsum[-1])
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    if layout == "nz":
+        wkw, wv = dict(weight_nz=(t(_to_nz(np.ascontiguousarray(wt.transpose(0, 2, 1)))), "nz5d")), None
+    else:
+        wkw, wv = {}, [_weight_views(wt, dev, layout)]
+    acc = aclnn.grouped_matmul_v4([t(x)], wv, group_list=t(cumsum), split_item=3, group_type=0, **wkw)[0]
+    y = aclnn.grouped_matmul_v4([t(x)], wv, scale=[t(scale)], per_token_scale=[t(pt)], group_list=t(cumsum), split_item=3,
+                                group_type=0, output_dtype=torch.bfloat16, **wkw)[0]
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True))
+    ref = oracle.grouped_matmul_dequant(x, wt, scale, pt, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), ref)
