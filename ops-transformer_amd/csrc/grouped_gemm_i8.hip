@@ -327,33 +327,41 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
             for (int mi = 0; mi < kSubM; ++mi) {
                 const int rTop = waveRow0 + 32 * mi;
                 if (mi >= mySub || rTop >= rows) continue;
-                // Whole MFMA tiles (wave-uniform test) take a copy of the loop with no row checks: a per-lane check
-                // makes every element a predicated basic block of its own, and the sixteen independent chains of a
-                // tile no longer interleave.
-                auto rowsOfTile = [&](auto fullTag) __attribute__((always_inline)) {
+                // The row checks are made per group of eight rows (accumulator entries 4q .. 4q + 3 of the two lane
+                // halves), wave-uniformly: a group wholly inside the expert's rows takes a copy of the code without
+                // checks, a group wholly outside is skipped, and only the one group that straddles the last row tests
+                // every lane.  A per-lane test makes every element a predicated basic block of its own, and the
+                // independent chains of a tile no longer interleave.
+                auto rowGroup = [&](int q, auto fullTag) __attribute__((always_inline)) {
                     constexpr bool kFull = decltype(fullTag)::value;
+                    float4 rs = make_float4(1.0f, 1.0f, 1.0f, 1.0f);  // multiplying by 1 is exact
+                    if (hasRowScale) rs = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
+                    const float rsv[4] = {rs.x, rs.y, rs.z, rs.w};
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        float4 rs = make_float4(1.0f, 1.0f, 1.0f, 1.0f);  // multiplying by 1 is exact
-                        if (hasRowScale) rs = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
-                        const float rsv[4] = {rs.x, rs.y, rs.z, rs.w};
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int v = 4 * q + i;
-                            const Float2 f = {__fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), sc0), rsv[i]),
-                                              __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), sc1), rsv[i])};
-                            const uint32_t pk = toBf16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2))
-                                                       : (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[0]))) |
-                                                          (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[1]))) << 16));
-                            const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
-                            const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
-                            uint16_t* const rowPtr = outTile + static_cast<int64_t>(32 * mi + 8 * q + i) * a.N;
-                            if (kFull || rTop + 8 * q + 4 * lhi + i < rows) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t*>(rowPtr + laneOff));
-                        }
+                    for (int i = 0; i < 4; ++i) {
+                        const int v = 4 * q + i;
+                        const Float2 f = {__fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), sc0), rsv[i]),
+                                          __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), sc1), rsv[i])};
+                        const uint32_t pk = toBf16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2))
+                                                   : (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[0]))) |
+                                                      (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[1]))) << 16));
+                        const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
+                        const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
+                        uint16_t* const rowPtr = outTile + static_cast<int64_t>(32 * mi + 8 * q + i) * a.N;
+                        if (kFull || rTop + 8 * q + 4 * lhi + i < rows) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t*>(rowPtr + laneOff));
                     }
                 };
-                if (rTop + 32 <= rows) rowsOfTile(std::true_type{});
-                else rowsOfTile(std::false_type{});
+                if (rTop + 32 <= rows) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) rowGroup(q, std::true_type{});
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (rTop + 8 * q >= rows) break;
+                        if (rTop + 8 * q + 8 <= rows) rowGroup(q, std::true_type{});
+                        else rowGroup(q, std::false_type{});
+                    }
+                }
             }
             return;
         }
@@ -439,29 +447,38 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                 float* const sTile = a.sOut + static_cast<int64_t>(rowBase + rTop) * a.halfN;
                 const int32_t laneOff = 4 * lhi * a.halfN + j;
                 float m[16];
-                // Whole MFMA tiles (wave-uniform test) take a copy of the loop with no row checks: a per-lane check
-                // makes every element a predicated basic block of its own, and the sixteen independent
-                // exp / reciprocal chains of a tile no longer interleave.
-                auto rowsOfTile = [&](auto fullTag) __attribute__((always_inline)) {
+                // Row checks per group of eight rows, wave-uniformly, as in the 16-bit stores above.
+                auto rowGroup = [&](int q, auto fullTag) __attribute__((always_inline)) {
                     constexpr bool kFull = decltype(fullTag)::value;
+                    const float4 xs4 = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
+                    const float xsv[4] = {xs4.x, xs4.y, xs4.z, xs4.w};
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const float4 xs4 = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
-                        const float xsv[4] = {xs4.x, xs4.y, xs4.z, xs4.w};
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int v = 4 * q + i;
-                            const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), xsv[i]), scA);
-                            const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xsv[i]), scB);
-                            float sv = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
-                            const bool ok = kFull || rTop + 8 * q + 4 * lhi + i < rows;
-                            if (ok) __builtin_nontemporal_store(sv, &sTile[static_cast<int64_t>(8 * q + i) * a.halfN + laneOff]);
-                            m[v] = ok ? fabsf(sv) : 0.0f;
-                        }
+                    for (int i = 0; i < 4; ++i) {
+                        const int v = 4 * q + i;
+                        const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), xsv[i]), scA);
+                        const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xsv[i]), scB);
+                        float sv = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
+                        const bool ok = kFull || rTop + 8 * q + 4 * lhi + i < rows;
+                        if (ok) __builtin_nontemporal_store(sv, &sTile[static_cast<int64_t>(8 * q + i) * a.halfN + laneOff]);
+                        m[v] = ok ? fabsf(sv) : 0.0f;
                     }
                 };
-                if (rTop + 32 <= rows) rowsOfTile(std::true_type{});
-                else rowsOfTile(std::false_type{});
+                if (rTop + 32 <= rows) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) rowGroup(q, std::true_type{});
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (rTop + 8 * q >= rows) {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) m[4 * q + i] = 0.0f;
+                        } else if (rTop + 8 * q + 8 <= rows) {
+                            rowGroup(q, std::true_type{});
+                        } else {
+                            rowGroup(q, std::false_type{});
+                        }
+                    }
+                }
                 // lanes l and l ^ 16: one instruction trades the upper-row half of m[i] for the lower-row half of
                 // m[i + 8]; afterwards lanes 0..15 of each half-wave own v = i and lanes 16..31 own v = i + 8
                 typedef unsigned int Uint2 __attribute__((ext_vector_type(2)));
