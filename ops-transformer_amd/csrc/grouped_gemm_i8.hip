@@ -274,6 +274,15 @@ __device__ __forceinline__ float LoadScale(const void* p, int64_t i, int dtype) 
     return __uint_as_float(static_cast<uint32_t>(raw) << 16);
 }
 
+// fp32 -> fp16, round to nearest even, of a value that is itself an fp32 result.  The reference rounds its products to
+// fp32 and then casts; left in sight of each other, a multiply and this conversion are merged by the compiler into one
+// v_fma_mixlo_f16, which rounds the exact product once -- a different value in the rare double-rounding cases.  The
+// empty statement hides the value's origin.
+__device__ __forceinline__ uint16_t HalfBitsOfRounded(float f) {
+    asm("" : "+v"(f));
+    return __half_as_ushort(__float2half_rn(f));
+}
+
 // Byte offset of (channel n, k = 0) inside one expert's weights; consecutive k are a.wStrideK bytes apart (32 in the
 // blocked layout: a 32-channel block holds its K rows of 32 channel bytes back to back).
 __device__ __forceinline__ int64_t WeightRowBase(const KernelArgs& a, int32_t n) {
@@ -332,36 +341,51 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                 // checks, a group wholly outside is skipped, and only the one group that straddles the last row tests
                 // every lane.  A per-lane test makes every element a predicated basic block of its own, and the
                 // independent chains of a tile no longer interleave.
-                auto rowGroup = [&](int q, auto fullTag) __attribute__((always_inline)) {
+                // the tile's 32 row scales, read in one go (one wave-uniform test instead of one per row group)
+                float4 rsTile[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) rsTile[q] = make_float4(1.0f, 1.0f, 1.0f, 1.0f);  // multiplying by 1 is exact
+                if (hasRowScale) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) rsTile[q] = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
+                }
+                auto rowGroup = [&](int q, auto fullTag, auto bf16Tag) __attribute__((always_inline)) {
                     constexpr bool kFull = decltype(fullTag)::value;
-                    float4 rs = make_float4(1.0f, 1.0f, 1.0f, 1.0f);  // multiplying by 1 is exact
-                    if (hasRowScale) rs = *reinterpret_cast<const float4*>(ldsRowScale + rTop + 8 * q + 4 * lhi);
+                    constexpr bool kToBf16 = decltype(bf16Tag)::value;  // compile-time: a run-time choice per element splits the block
+                    const float4 rs = rsTile[q];
                     const float rsv[4] = {rs.x, rs.y, rs.z, rs.w};
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int v = 4 * q + i;
                         const Float2 f = {__fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), sc0), rsv[i]),
                                           __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), sc1), rsv[i])};
-                        const uint32_t pk = toBf16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2))
-                                                   : (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[0]))) |
-                                                      (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f[1]))) << 16));
+                        uint32_t pk;
+                        if constexpr (kToBf16) {
+                            pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));
+                        } else {
+                            pk = static_cast<uint32_t>(HalfBitsOfRounded(f[0])) | (static_cast<uint32_t>(HalfBitsOfRounded(f[1])) << 16);
+                        }
                         const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(pk), 0xB1, 0xF, 0xF, true));
                         const uint32_t word = __builtin_amdgcn_perm(got, pk, oddLane ? 0x03020706u : 0x05040100u);
                         uint16_t* const rowPtr = outTile + static_cast<int64_t>(32 * mi + 8 * q + i) * a.N;
                         if (kFull || rTop + 8 * q + 4 * lhi + i < rows) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t*>(rowPtr + laneOff));
                     }
                 };
-                if (rTop + 32 <= rows) {
+                auto rowsOfTile = [&](auto bf16Tag) __attribute__((always_inline)) {
+                    if (rTop + 32 <= rows) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) rowGroup(q, std::true_type{});
-                } else {
+                        for (int q = 0; q < 4; ++q) rowGroup(q, std::true_type{}, bf16Tag);
+                    } else {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        if (rTop + 8 * q >= rows) break;
-                        if (rTop + 8 * q + 8 <= rows) rowGroup(q, std::true_type{});
-                        else rowGroup(q, std::false_type{});
+                        for (int q = 0; q < 4; ++q) {
+                            if (rTop + 8 * q >= rows) break;
+                            if (rTop + 8 * q + 8 <= rows) rowGroup(q, std::true_type{}, bf16Tag);
+                            else rowGroup(q, std::false_type{}, bf16Tag);
+                        }
                     }
-                }
+                };
+                if (toBf16) rowsOfTile(std::true_type{});
+                else rowsOfTile(std::false_type{});
             }
             return;
         }
@@ -411,8 +435,7 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                     const Float2 f = {y0, y1};
                     pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));  // v_cvt_pk_bf16_f32
                 } else {
-                    pk = static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y0))) |
-                         (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y1))) << 16);
+                    pk = static_cast<uint32_t>(HalfBitsOfRounded(y0)) | (static_cast<uint32_t>(HalfBitsOfRounded(y1)) << 16);
                 }
                 if (pairStores) {
                     // quad_perm [1,0,3,2]: exchange with the lane whose index differs in bit 0, then keep
@@ -1183,7 +1206,7 @@ struct RequantArgs {
 };
 
 __device__ __forceinline__ int8_t QuantOne(float s, float inv) {
-    const __half h = __float2half_rn(__fmul_rn(s, inv));
+    const __half h = __ushort_as_half(HalfBitsOfRounded(__fmul_rn(s, inv)));
     return static_cast<int8_t>(__float2int_rn(__half2float(h)));
 }
 
