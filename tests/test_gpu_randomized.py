@@ -131,8 +131,13 @@ def test_grouped_gemm_random(aclnn, oracle, dev, seed):
         h, hs = aclnn.grouped_matmul_swiglu_quant(xd, wv, torch.from_numpy(cumsum).to(dev), torch.from_numpy(scale).to(dev),
                                                   torch.from_numpy(per_token).to(dev))
         torch.cuda.synchronize()
-        assert np.abs(h.cpu().numpy()[:covered].astype(np.int32) - h_r[:covered].astype(np.int32)).max(initial=0) <= 1
-        np.testing.assert_allclose(hs.cpu().numpy()[:covered], hs_r[:covered], rtol=1e-2)
+        # A row whose every |S| is below ~1e-30 exists only through denormal intermediates (swish of an argument below
+        # -87: the reciprocal of 1 + exp(87) is a denormal, which v_rcp_f32 returns as zero); the CPU oracle keeps
+        # denormals, the kernel makes such a row a zero row.  With 2 to 4 columns per row the sweep does meet one.
+        live = hs_r[:covered] > 1e-30
+        assert np.abs(h.cpu().numpy()[:covered][live].astype(np.int32) - h_r[:covered][live].astype(np.int32)).max(initial=0) <= 1
+        np.testing.assert_allclose(hs.cpu().numpy()[:covered][live], hs_r[:covered][live], rtol=1e-2)
+        assert (hs.cpu().numpy()[:covered][~live] <= 1e-30).all()
 
 
 @pytest.mark.parametrize("seed", SEEDS[:12])
