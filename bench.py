@@ -255,6 +255,11 @@ def _other_configs(pkg, dev, headline, steps, warmup):
         gc.collect()
         torch.cuda.empty_cache()
 
+    if headline.cfg.name.startswith("c1"):
+        # the headline's own pass replayed from a HIP graph, for comparison with the ten eager launches (a graph of long
+        # kernels need not replay faster than they launch: the decode pass gains from it, this one does not)
+        out["c1_graph"] = headline.summary(headline.measure(steps, warmup, graph=True), steps,
+                                           "HIP graph replay (kernel durations from eager passes)")
     if headline.cfg.name.startswith("c1") and headline.ffn.routing == "v3":
         v2 = headline.with_routing("v2")
         out["c1_v2_routed"] = v2.summary(v2.measure(steps, warmup), steps, "eager two-phase calls")
