@@ -95,6 +95,37 @@ def check_lds_dma_assembly(asm_path):
     return loads
 
 
+def check_ring_kernel_codegen(asm_path):
+    """Second build-time guard on the device assembly of grouped_gemm_i8.hip, for three properties of the generated code
+    that the kernels' speed and exactness rest on and that a compiler can change without any test noticing at once:
+      * no LDS-ring kernel (StreamGemmKernel) uses scratch memory -- a spilled register is reloaded inside the tile loop;
+      * no generic (flat) memory instruction: one still in flight makes the compiler drain vmcnt, DMAs included, in
+        front of every LDS read;
+      * no mixed-precision multiply-add (v_fma_mix*, v_mad_mix*): that is a product and its fp16 conversion merged into
+        one rounding, where the reference rounds the product to fp32 first.
+    Returns the number of ring kernels checked."""
+    text = open(asm_path).read()
+    for bad in ("v_fma_mix", "v_mad_mix"):
+        if bad in text:
+            raise RuntimeError("%s: the compiler merged a multiply with an fp16 conversion (%s*)" % (asm_path, bad))
+    for bad in ("flat_load_", "flat_store_", "flat_atomic_"):
+        if bad in text:
+            raise RuntimeError("%s: generic memory instruction (%s*) in the GEMM kernels" % (asm_path, bad))
+    checked = 0
+    for block in text.split(".amdhsa_kernel ")[1:]:
+        name = block.split()[0]
+        if "StreamGemmKernel" not in name:
+            continue
+        fields = dict(l.split()[:2] for l in block.split(".end_amdhsa_kernel")[0].splitlines()[1:] if len(l.split()) >= 2)
+        if int(fields.get(".amdhsa_private_segment_fixed_size", "0")) != 0:
+            raise RuntimeError("%s: %s spills %s bytes per lane to scratch" %
+                               (asm_path, name, fields[".amdhsa_private_segment_fixed_size"]))
+        checked += 1
+    if checked == 0:
+        raise RuntimeError("%s: no LDS-ring kernel found" % asm_path)
+    return checked
+
+
 def _headers():
     out = []
     for base in (CSRC, os.path.join(ROOT, "include")):
@@ -123,6 +154,7 @@ def _compile(src, force):
         stem = os.path.join(OBJ_DIR, os.path.splitext(src)[0])
         try:
             check_lds_dma_assembly(stem + "-hip-amdgcn-amd-amdhsa-gfx950.s")
+            check_ring_kernel_codegen(stem + "-hip-amdgcn-amd-amdhsa-gfx950.s")
         except Exception:
             os.remove(obj)  # never leave an object behind that the guard refused
             raise

@@ -1,5 +1,6 @@
-"""The two build-time guards of ops-transformer_amd/build.py around the LDS-DMA kernels: the compiler pin and the check
-that, in the device assembly, m0 is written only as the first half of an (s_mov_b32 m0, global_load_lds_dwordx4) pair."""
+"""The build-time guards of ops-transformer_amd/build.py around the LDS-DMA kernels: the compiler pin, the check that, in
+the device assembly, m0 is written only as the first half of an (s_mov_b32 m0, global_load_lds_dwordx4) pair, and the
+check of the generated code for scratch use, generic memory instructions and merged multiply-convert instructions."""
 import importlib.util
 import os
 
@@ -60,3 +61,35 @@ def test_compiler_pin(build, monkeypatch):
         build.check_compiler()
     monkeypatch.setenv("OPAPI_ALLOW_UNVALIDATED_COMPILER", "1")
     assert "roc-99" in build.check_compiler()
+
+
+CODEGEN_GOOD = """
+_ZN4gemm16StreamGemmKernelILi1ELi0EEEvv:
+	v_mul_f32_e32 v1, v2, v3
+	v_cvt_f16_f32_e32 v1, v1
+	global_load_dword v4, v[0:1], off
+	s_endpgm
+	.amdhsa_kernel _ZN4gemm16StreamGemmKernelILi1ELi0EEEvv
+		.amdhsa_private_segment_fixed_size 0
+		.amdhsa_next_free_vgpr 132
+	.end_amdhsa_kernel
+	.amdhsa_kernel _ZN4gemm13RequantKernelEv
+		.amdhsa_private_segment_fixed_size 0
+	.end_amdhsa_kernel
+"""
+
+
+def test_codegen_guard_accepts_clean_kernels(build, tmp_path):
+    assert build.check_ring_kernel_codegen(_write(tmp_path, CODEGEN_GOOD)) == 1
+
+
+@pytest.mark.parametrize("bad", [
+    CODEGEN_GOOD.replace(".amdhsa_private_segment_fixed_size 0\n\t\t.amdhsa_next", ".amdhsa_private_segment_fixed_size 48\n\t\t.amdhsa_next"),  # a ring kernel spills
+    CODEGEN_GOOD.replace("v_cvt_f16_f32_e32 v1, v1", "v_fma_mixlo_f16 v1, v2, v3, 0"),       # product and conversion merged
+    CODEGEN_GOOD.replace("global_load_dword v4, v[0:1], off", "flat_load_dword v4, v[0:1]"),  # a generic load
+    CODEGEN_GOOD.replace("StreamGemmKernel", "OtherKernel"),                                  # nothing to check
+])
+def test_codegen_guard_refuses(build, tmp_path, bad):
+    assert bad != CODEGEN_GOOD
+    with pytest.raises(RuntimeError):
+        build.check_ring_kernel_codegen(_write(tmp_path, bad))
