@@ -1281,9 +1281,9 @@ uint64_t* gSpanBuf[kSpanKinds] = {nullptr, nullptr, nullptr};
 int gSpanGrid[kSpanKinds] = {0, 0, 0};
 int gSpanTileM[kSpanKinds] = {0, 0, 0};
 
-// Device buffer for the next ring-kernel launch of this epilogue kind (allocated on first use, cleared on the stream),
-// or null when recording is off.
-uint64_t* SpanBufferFor(Epilogue epi, int grid, int tileM, hipStream_t stream) {
+// Device buffer for the next ring-kernel launch of this epilogue kind (allocated on first use; every workgroup of the
+// launch writes its own entry), or null when recording is off.
+uint64_t* SpanBufferFor(Epilogue epi, int grid, int tileM) {
     if (gSpansOn.load(std::memory_order_relaxed) == 0 || grid > kSpanMaxGrid) return nullptr;
     const int k = static_cast<int>(epi);
     if (gSpanBuf[k] == nullptr && hipMalloc(&gSpanBuf[k], kSpanMaxGrid * 3 * sizeof(uint64_t)) != hipSuccess) return nullptr;
@@ -1305,7 +1305,7 @@ hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t ma
     grid = grid / kXcds * kXcds;
     if (grid < kXcds) grid = kXcds;
     KernelArgs launchArgs = args;
-    launchArgs.wgSpans = SpanBufferFor(kEpi, static_cast<int>(grid), Cfg::kTileM, stream);
+    launchArgs.wgSpans = SpanBufferFor(kEpi, static_cast<int>(grid), Cfg::kTileM);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, launchArgs, sched);
     return hipGetLastError();
 }
