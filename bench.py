@@ -116,39 +116,52 @@ def _recorded_traffic(config_name):
     return value, src
 
 
-def _gate_up_roofline(cfg, touched, kernels):
-    """Roofline block of the gate/up grouped GEMM from the library's event timer.
-
-    Algorithmic bytes of one launch: the touched experts' gate/up weights and channel scales, the expanded int8 rows
-    and their scales in, the int8 activations and their scales out.  Algorithmic ops: 4 * M * H * I."""
-    M, H, I = cfg.tokens * cfg.top_k, cfg.hidden, cfg.inter
-    gemm1_bytes = touched * 2 * H * I + touched * 2 * I * 4 + M * H + M * 4 + M * I + M * 4
-    gemm1_ops = 4 * M * H * I
-    n1, total1 = kernels.get("gmm_swiglu", (0, 0.0))
-    gemm1_ms = total1 / max(n1, 1)
-    hbm_frac = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if gemm1_ms > 0 else None
-    mfma_frac = gemm1_ops / (gemm1_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS if gemm1_ms > 0 else None
-    # bound of the kernel at this shape: time at HBM peak vs time at MFMA peak
-    t_hbm = gemm1_bytes / (HBM_PEAK_GBS * 1e9)
-    t_mfma = gemm1_ops / (INT8_PEAK_TOPS * 1e12)
-    traffic, traffic_source = _recorded_traffic(cfg.name)
+def _kernel_roofline(name, kernel, timer_name, nbytes, ops, kernels, traffic=None, traffic_source=None):
+    """Roofline block of one grouped GEMM kernel from the library's event timer: both fractions, and as `bound` the
+    roof that is the lower one for the kernel's algorithmic bytes and ops."""
+    n, total = kernels.get(timer_name, (0, 0.0))
+    ms = total / max(n, 1)
+    hbm_frac = nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if ms > 0 else None
+    mfma_frac = ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS if ms > 0 else None
+    t_hbm = nbytes / (HBM_PEAK_GBS * 1e9)
+    t_mfma = ops / (INT8_PEAK_TOPS * 1e12)
     if t_hbm >= t_mfma:
-        roofline = {"bound": "hbm", "achieved": gemm1_bytes / (gemm1_ms * 1e-3) / 1e9 if gemm1_ms else None,
+        roofline = {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9 if ms else None,
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac, "traffic": traffic}
     else:
-        roofline = {"bound": "mfma", "achieved": gemm1_ops / (gemm1_ms * 1e-3) / 1e12 if gemm1_ms else None,
+        roofline = {"bound": "mfma", "achieved": ops / (ms * 1e-3) / 1e12 if ms else None,
                     "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": traffic}
-    roofline.update({"traffic_source": traffic_source,
-                     "kernel": "StreamGemmKernel<..., kSwiglu> (gate/up GEMM + SwiGLU; timer name gmm_swiglu)",
-                     "kernel_ms": gemm1_ms, "algorithmic_bytes": gemm1_bytes, "algorithmic_ops": gemm1_ops,
-                     "hbm_frac": hbm_frac, "mfma_frac": mfma_frac})
+    if traffic_source is not None:
+        roofline["traffic_source"] = traffic_source
+    roofline.update({"kernel": kernel, "kernel_ms": ms, "launches_timed": n, "algorithmic_bytes": nbytes,
+                     "algorithmic_ops": ops, "hbm_frac": hbm_frac, "mfma_frac": mfma_frac,
+                     "time_at_hbm_peak_ms": t_hbm * 1e3, "time_at_mfma_peak_ms": t_mfma * 1e3})
     return roofline
+
+
+def _gate_up_roofline(cfg, touched, kernels):
+    """Gate/up grouped GEMM.  Algorithmic bytes of one launch: the touched experts' gate/up weights and channel scales,
+    the expanded int8 rows and their scales in, the int8 activations and their scales out.  Ops: 4 * M * H * I."""
+    M, H, I = cfg.tokens * cfg.top_k, cfg.hidden, cfg.inter
+    nbytes = touched * 2 * H * I + touched * 2 * I * 4 + M * H + M * 4 + M * I + M * 4
+    traffic, traffic_source = _recorded_traffic(cfg.name)
+    return _kernel_roofline("gate_up", "StreamGemmKernel<..., kSwiglu> (gate/up GEMM + SwiGLU; timer name gmm_swiglu)",
+                            "gmm_swiglu", nbytes, 4 * M * H * I, kernels, traffic, traffic_source)
+
+
+def _down_roofline(cfg, touched, kernels):
+    """Down-projection grouped GEMM.  Algorithmic bytes of one launch: the touched experts' down weights and channel
+    scales, the int8 activations and their scales in, the bf16 rows out.  Ops: 2 * M * H * I."""
+    M, H, I = cfg.tokens * cfg.top_k, cfg.hidden, cfg.inter
+    nbytes = touched * H * I + touched * H * 4 + M * I + M * 4 + M * H * 2
+    return _kernel_roofline("down", "StreamGemmKernel<..., kDequant> (down GEMM + dequant; timer name gmm_dequant)",
+                            "gmm_dequant", nbytes, 2 * M * H * I, kernels)
 
 
 class Workload:
     """One configuration resident on the GPU: routing inputs, quantised activations, expert weights, the chain."""
 
-    def __init__(self, pkg, cfg, dev, routing="v3", **ffn_kwargs):
+    def __init__(self, pkg, cfg, dev, routing="v2", **ffn_kwargs):
         import torch
         self.pkg, self.cfg, self.dev = pkg, cfg, dev
         seed = pkg.synth.CONFIGS.index(cfg)
@@ -168,15 +181,16 @@ class Workload:
         other.ffn = self.pkg.MoeFfnW8A8(*self.weights, routing=routing, **self.ffn_kwargs)
         return other
 
-    def measure(self, steps, warmup, graph=False):
-        """Times `steps` passes (after `warmup` untimed ones) between two device synchronisations, then runs `steps`
-        further eager passes with the library's HIP-event timer on for the per-kernel durations.
+    def measure(self, steps, warmup, graph=False, repeats=5):
+        """Times `steps` passes (after `warmup` untimed ones) as `repeats` consecutive blocks, each between two device
+        synchronisations with nothing else in the stream; the figure reported per pass is the median block (minimum,
+        maximum and the mean over all `steps` passes are kept beside it).  Then runs min(steps, 20) further eager passes
+        with the library's HIP-event timer on for the per-kernel durations.
 
         The timer brackets every kernel launch with a pair of events on the launch stream; on this runtime each pair
         costs the stream about 10 us between kernels (0.08 ms over the eight launches of a decode pass), so the passes
         that give tokens/s run with the timer off and the passes that give the kernel durations follow immediately, in
-        the same process, on the same buffers.  Returns (seconds per pass, {kernel name: (launches, total ms)},
-        seconds per pass with the timer on)."""
+        the same process, on the same buffers."""
         import torch
         aclnn = self.pkg.aclnn
         args = (self.d_xq, self.d_xs, self.d_idx, self.d_wgt)
@@ -187,30 +201,39 @@ class Workload:
             step = lambda: self.ffn.forward(*args)
         for _ in range(warmup):
             step()
+        repeats = max(1, min(repeats, steps))
+        blocks = [len(b) for b in np.array_split(np.arange(steps), repeats)]
+        per_pass = []
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            step()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
+        t_all = time.perf_counter()
+        for n in blocks:
+            t0 = time.perf_counter()
+            for _ in range(n):
+                step()
+            torch.cuda.synchronize()
+            per_pass.append((time.perf_counter() - t0) / n)
+        elapsed = time.perf_counter() - t_all
+        timer_steps = min(steps, 20)
         aclnn.kernel_timer_enable(True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for _ in range(timer_steps):
             self.ffn.forward(*args)
         torch.cuda.synchronize()
         elapsed_timer = time.perf_counter() - t0
         kernels = aclnn.kernel_timer_report()
         aclnn.kernel_timer_enable(False)
-        # how evenly the static deal of GEMM tiles ends on the eight XCDs: one more pass with span recording on
+        # how evenly the deal of GEMM tiles ends on the eight XCDs: one more pass with span recording on
         aclnn.gemm_workgroup_spans_enable(True)
         self.ffn.forward(*args)
         self.spans = aclnn.gemm_workgroup_spans_report()
         aclnn.gemm_workgroup_spans_enable(False)
-        return elapsed / steps, kernels, elapsed_timer / steps
+        return {"sec_per_pass": float(np.median(per_pass)), "sec_min": min(per_pass), "sec_max": max(per_pass),
+                "sec_mean": elapsed / steps, "blocks": blocks, "kernels": kernels, "timer_steps": timer_steps,
+                "sec_with_timer": elapsed_timer / timer_steps}
 
     def summary(self, measured, steps, launch):
-        sec_per_pass, kernels, sec_with_timer = measured
+        sec_per_pass, kernels, sec_with_timer = measured["sec_per_pass"], measured["kernels"], measured["sec_with_timer"]
         cfg = self.cfg
         work = self.pkg.synth.algorithmic_work(cfg, self.touched)
         return {
@@ -221,13 +244,19 @@ class Workload:
             "launch": launch,
             "experts_touched": self.touched,
             "ms_per_step": sec_per_pass * 1e3,
+            "ms_per_step_repeats": {"blocks_of_passes": measured["blocks"], "statistic": "median of the blocks",
+                                    "min": measured["sec_min"] * 1e3, "max": measured["sec_max"] * 1e3,
+                                    "mean_over_all_passes": measured["sec_mean"] * 1e3},
             "ms_per_step_kernel_timer_on": sec_with_timer * 1e3,
             "tokens_per_s": cfg.tokens / sec_per_pass,
             "end_to_end": {"mfma_frac": work["ops"] / sec_per_pass / 1e12 / INT8_PEAK_TOPS,
                            "hbm_frac": work["bytes"] / sec_per_pass / 1e9 / HBM_PEAK_GBS,
                            "algorithmic_ops": work["ops"], "algorithmic_bytes": work["bytes"]},
-            "kernels_ms": {k: v[1] / float(steps) for k, v in sorted(kernels.items())},
+            "kernels_ms": {k: v[1] / float(measured["timer_steps"]) for k, v in sorted(kernels.items())},
             "roofline": _gate_up_roofline(cfg, self.touched, kernels),
+            "roofline_down_gemm": _down_roofline(cfg, self.touched, kernels),
+            "workspace_bytes": dict(self.ffn.workspace.requested, allocated=int(self.ffn.workspace.tensor.numel())
+                                    if self.ffn.workspace.tensor is not None else 0),
             "gemm_tile_balance": self._tile_balance(),
         }
 
@@ -260,15 +289,18 @@ def _other_configs(pkg, dev, headline, steps, warmup):
         # kernels need not replay faster than they launch: the decode pass gains from it, this one does not)
         out["c1_graph"] = headline.summary(headline.measure(steps, warmup, graph=True), steps,
                                            "HIP graph replay (kernel durations from eager passes)")
-    if headline.cfg.name.startswith("c1") and headline.ffn.routing == "v3":
-        v2 = headline.with_routing("v2")
-        out["c1_v2_routed"] = v2.summary(v2.measure(steps, warmup), steps, "eager two-phase calls")
-        del v2
+    if headline.cfg.name.startswith("c1"):
+        # the same tensors behind the other routing operator (one aclnnMoeInitRoutingV3 call instead of the two
+        # aclnnMoeInitRoutingV2 calls, or the other way round)
+        name = "v3" if headline.ffn.routing == "v2" else "v2"
+        alt = headline.with_routing(name)
+        out["c1_%s_routed" % name] = alt.summary(alt.measure(steps, warmup), steps, "eager two-phase calls")
+        del alt
     for name in ("c3", "c2", "c4"):
         if headline.cfg.name.startswith(name):
             continue
         release()
-        w = Workload(pkg, pkg.synth.config(name), dev)
+        w = Workload(pkg, pkg.synth.config(name), dev, routing=headline.ffn.routing)
         out[name] = w.summary(w.measure(steps, warmup), steps, "eager two-phase calls")
         if name == "c3":
             out["c3_graph"] = w.summary(w.measure(steps, warmup, graph=True), steps,
@@ -281,7 +313,9 @@ def _other_configs(pkg, dev, headline, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="the timed passes run as this many blocks, each between two synchronisations; ms_per_step is the median block")
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -290,8 +324,9 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true")
     ap.add_argument("--graph", action="store_true",
                     help="replay the pass from a HIP graph (second phases only) instead of calling the operators eagerly")
-    ap.add_argument("--routing", choices=("v2", "v3"), default="v3",
-                    help="routing operator at the head of the chain: aclnnMoeInitRoutingV3 (default) or V2")
+    ap.add_argument("--routing", choices=("v2", "v3"), default="v2",
+                    help="routing operator at the head of the chain: aclnnMoeInitRoutingV2 (default, two calls: rows and "
+                         "scale column) or aclnnMoeInitRoutingV3 (one call)")
     ap.add_argument("--weight-nz", action="store_true",
                     help="give the GEMM operators FRACTAL_NZ weights ([E, N/32, K/16, 16, 32]) instead of transposed views")
     ap.add_argument("--weight-row-major", action="store_true",
@@ -316,8 +351,8 @@ def main():
 
     head = Workload(pkg, cfg, dev, routing=args.routing, fused_combine=args.fused_combine, weight_nz=args.weight_nz,
                     weight_row_major=args.weight_row_major)
-    measured = head.measure(args.steps, args.warmup, graph=args.graph)
-    sec_per_pass = measured[0]
+    measured = head.measure(args.steps, args.warmup, graph=args.graph, repeats=args.repeats)
+    sec_per_pass = measured["sec_per_pass"]
     if args.calibration_copy:
         src = torch.empty(1 << 30, dtype=torch.int8, device=dev).fill_(3)
         dst = torch.empty_like(src)
@@ -336,6 +371,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": s["ms_per_step"],
+        "ms_per_step_repeats": s["ms_per_step_repeats"],
         "ms_per_step_kernel_timer_on": s["ms_per_step_kernel_timer_on"],
         "higher_is_better": True,
         "scaling": "weak",
@@ -351,6 +387,8 @@ def main():
         "end_to_end": dict(s["end_to_end"], tops=work["ops"] / sec_per_pass / 1e12, gbps=work["bytes"] / sec_per_pass / 1e9),
         "kernels_ms": s["kernels_ms"],
         "roofline": s["roofline"],
+        "roofline_down_gemm": s["roofline_down_gemm"],
+        "workspace_bytes": s["workspace_bytes"],
         "gemm_tile_balance": s["gemm_tile_balance"],
     }
     # what the matrix pipe sustains with nothing else going on: the clock under matrix load follows the switching
@@ -367,7 +405,7 @@ def main():
         result["cpu_baseline"] = {"value": v, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
                                   "sample": desc}
     if not args.no_other_configs:
-        result["other_configs"] = _other_configs(pkg, dev, head, steps=min(args.steps, 10), warmup=min(args.warmup, 2))
+        result["other_configs"] = _other_configs(pkg, dev, head, steps=min(args.steps, 20), warmup=min(args.warmup, 2))
     print(json.dumps(result))
 
 

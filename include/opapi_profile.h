@@ -53,6 +53,9 @@ __attribute__((visibility("default"))) int opapiInt8MfmaRateProbe(int uniformRan
  * workgroups (hence to the eight XCDs) ends.  While on, every workgroup of a ring-kernel launch records when it started
  * and ended (the GPU's 100 MHz real-time counter) and how many tiles it computed; only the last launch of each kind
  * (gmm_swiglu, gmm_dequant, gmm_int32) is kept.  Off by default; costs one branch per workgroup when off.
+ * Turning it on allocates three 24 KB device buffers on the current device (once; kept until the process ends) -- the
+ * launch paths themselves never allocate -- and discards earlier records; launches on another device, or of more than
+ * 1024 workgroups, are not recorded and drop their kind's record.  One launching thread at a time.
  */
 __attribute__((visibility("default"))) void opapiGemmWorkgroupSpansEnable(int enable);
 

@@ -209,8 +209,11 @@ class Workspace:
 
     def __init__(self):
         self.tensor = None
+        self.requested = {}  # operator name -> largest workspace size its first phase has asked for
 
-    def reserve(self, nbytes, device):
+    def reserve(self, nbytes, device, api=None):
+        if api is not None:
+            self.requested[api] = max(self.requested.get(api, 0), int(nbytes))
         if self.tensor is None or self.tensor.numel() < nbytes:
             self.tensor = torch.empty(nbytes, dtype=torch.uint8, device=device)
         return self.tensor
@@ -238,6 +241,8 @@ def _run_two_phase(api, args, device, workspace=None, static_workspace_api=None)
         return None
     ws_ptr = None
     ws_keepalive = None
+    if workspace is not None:
+        workspace.requested[api] = max(workspace.requested.get(api, 0), int(ws_size.value))
     if ws_size.value > 0:
         if workspace is not None:
             ws_keepalive = workspace.reserve(ws_size.value, device)

@@ -31,7 +31,9 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "opapi_common.h"
 
@@ -1274,19 +1276,29 @@ int DeviceCuCount() {
 }
 
 // ---- workgroup spans (opapiGemmWorkgroupSpans*, include/opapi_profile.h): a measurement aid, off by default ----
+// The buffers are allocated by opapiGemmWorkgroupSpansEnable(1) on the device that is current then, never on a launch
+// path; recording is for one device and one launching thread at a time (the mutex only keeps the bookkeeping whole).
 constexpr int kSpanKinds = 3;        // indexed by Epilogue
 constexpr int kSpanMaxGrid = 1024;
-std::atomic<int> gSpansOn{0};
+std::mutex gSpanMutex;
+bool gSpansOn = false;
+int gSpanDevice = -1;
 uint64_t* gSpanBuf[kSpanKinds] = {nullptr, nullptr, nullptr};
-int gSpanGrid[kSpanKinds] = {0, 0, 0};
+int gSpanGrid[kSpanKinds] = {0, 0, 0};   // workgroups of the last recorded launch of the kind; 0: nothing recorded
 int gSpanTileM[kSpanKinds] = {0, 0, 0};
 
-// Device buffer for the next ring-kernel launch of this epilogue kind (allocated on first use; every workgroup of the
-// launch writes its own entry), or null when recording is off.
+// Device buffer for the next ring-kernel launch of this epilogue kind (every workgroup of the launch writes its own
+// entry), or null when recording is off, the launch runs on another device or its grid exceeds the buffer -- the kind's
+// earlier record is dropped then, so that a report never shows another launch's figures as the last one's.
 uint64_t* SpanBufferFor(Epilogue epi, int grid, int tileM) {
-    if (gSpansOn.load(std::memory_order_relaxed) == 0 || grid > kSpanMaxGrid) return nullptr;
+    std::lock_guard<std::mutex> lock(gSpanMutex);
+    if (!gSpansOn) return nullptr;
     const int k = static_cast<int>(epi);
-    if (gSpanBuf[k] == nullptr && hipMalloc(&gSpanBuf[k], kSpanMaxGrid * 3 * sizeof(uint64_t)) != hipSuccess) return nullptr;
+    int dev = -1;
+    if (gSpanBuf[k] == nullptr || grid > kSpanMaxGrid || hipGetDevice(&dev) != hipSuccess || dev != gSpanDevice) {
+        gSpanGrid[k] = 0;
+        return nullptr;
+    }
     gSpanGrid[k] = grid;
     gSpanTileM[k] = tileM;
     return gSpanBuf[k];
@@ -1330,11 +1342,6 @@ hipError_t LaunchStreamShape(const Plan& plan, const KernelArgs& args, const int
     if (args.wNz) return LaunchStreamShapeOf<kEpi, true, false>(plan, args, sched, stream);
     if (args.wStrideN == 1) return LaunchStreamShapeOf<kEpi, false, true>(plan, args, sched, stream);  // row-major [K, N]
     return LaunchStreamShapeOf<kEpi, false, false>(plan, args, sched, stream);
-}
-
-template <Epilogue kEpi>
-hipError_t LaunchFast(const Plan& plan, const KernelArgs& args, const int32_t* sched, hipStream_t stream) {
-    return LaunchStreamShape<kEpi>(plan, args, sched, stream);
 }
 
 template <Epilogue kEpi>
@@ -1474,15 +1481,15 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
                                  : p.combineIndex != nullptr ? "gmm_combine" : "gmm_dequant", stream);
         switch (p.epilogue) {
             case Epilogue::kInt32:
-                e = fast ? LaunchFast<Epilogue::kInt32>(plan, ka, sched, stream)
+                e = fast ? LaunchStreamShape<Epilogue::kInt32>(plan, ka, sched, stream)
                          : LaunchGenericShape<Epilogue::kInt32>(plan, ka, sched, stream);
                 break;
             case Epilogue::kDequant:
-                e = fast ? LaunchFast<Epilogue::kDequant>(plan, ka, sched, stream)
+                e = fast ? LaunchStreamShape<Epilogue::kDequant>(plan, ka, sched, stream)
                          : LaunchGenericShape<Epilogue::kDequant>(plan, ka, sched, stream);
                 break;
             case Epilogue::kSwiglu:
-                e = fast ? LaunchFast<Epilogue::kSwiglu>(plan, ka, sched, stream)
+                e = fast ? LaunchStreamShape<Epilogue::kSwiglu>(plan, ka, sched, stream)
                          : LaunchGenericShape<Epilogue::kSwiglu>(plan, ka, sched, stream);
                 break;
         }
@@ -1500,13 +1507,32 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
 }  // namespace gemm
 
 extern "C" __attribute__((visibility("default"))) void opapiGemmWorkgroupSpansEnable(int enable) {
-    gemm::gSpansOn.store(enable ? 1 : 0, std::memory_order_relaxed);
+    using namespace gemm;
+    std::lock_guard<std::mutex> lock(gSpanMutex);
+    gSpansOn = false;
+    for (int k = 0; k < kSpanKinds; ++k) gSpanGrid[k] = 0;  // records of an earlier recording period are not reported
+    if (!enable) return;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    if (dev != gSpanDevice) {
+        // buffers of another device stay allocated until the process ends (a few KB); this device gets its own
+        for (int k = 0; k < kSpanKinds; ++k) gSpanBuf[k] = nullptr;
+        gSpanDevice = dev;
+    }
+    for (int k = 0; k < kSpanKinds; ++k) {
+        if (gSpanBuf[k] == nullptr && hipMalloc(&gSpanBuf[k], kSpanMaxGrid * 3 * sizeof(uint64_t)) != hipSuccess) {
+            gSpanBuf[k] = nullptr;
+            return;
+        }
+    }
+    gSpansOn = true;
 }
 
 extern "C" __attribute__((visibility("default"))) int opapiGemmWorkgroupSpansReport(char* buf, size_t cap) {
     using namespace gemm;
     if (buf == nullptr || cap == 0) return -1;
     if (hipDeviceSynchronize() != hipSuccess) return -1;
+    std::lock_guard<std::mutex> lock(gSpanMutex);
     static const char* const kNames[kSpanKinds] = {"gmm_int32", "gmm_dequant", "gmm_swiglu"};
     size_t used = 0;
     int lines = 0;

@@ -1,17 +1,19 @@
 """The quantized MoE expert FFN as a chain of the four aclnn operators (the caller side of the path).
 
-    aclnnMoeInitRoutingV3 -> aclnnGroupedMatmulSwigluQuant -> aclnnGroupedMatmulV4 -> aclnnMoeFinalizeRoutingV2
+    aclnnMoeInitRoutingV2 -> aclnnGroupedMatmulSwigluQuant -> aclnnGroupedMatmulV4 -> aclnnMoeFinalizeRoutingV2
 
 The reference has no in-repo code that chains them; real callers (torch_npu, vLLM-Ascend) do what ``forward`` does.
 Glue between the operators:
-  * activations arrive already quantized per token (int8 rows + fp32 scale); one MoeInitRoutingV3 call (quantMode -1,
-    INT8 x as this build's extension) routes the rows and carries the per-token scales along as expandedScale
-    (a row gather commutes with per-row quantization bit-exactly);
-  * routing emits the int64 cumsum (expertTokensNumType 0) both GEMM operators take as groupList;
-  * MoeFinalizeRoutingV2 is called with dropPadMode 2 because the scatter-type index (rowIdxType 1) is the row
-    arrangement expandedRowIdx[n*K + k] = destination.
-``routing="v2"`` keeps the older chain: MoeInitRoutingV2 on the rows plus a second MoeInitRoutingV2 call on the
-[T, 1] scale column, int32 cumsum.
+  * activations arrive already quantized per token (int8 rows + fp32 scale); MoeInitRoutingV2 routes the int8 rows
+    (INT8 x is this build's extension: a row gather commutes with per-row quantization bit-exactly) and a second
+    MoeInitRoutingV2 call routes the [T, 1] column of per-token scales the same way;
+  * routing emits the int32 cumsum (expertTokensCountOrCumsumFlag 1), which both GEMM operators take as groupList (the
+    reference wants int64 there; int32 is accepted as an extension, so no cast kernel sits between the operators);
+  * MoeFinalizeRoutingV2 is called with dropPadMode 2 because V2's index is the row arrangement
+    expandedRowIdx[n*K + k] = destination.
+``routing="v3"`` puts aclnnMoeInitRoutingV3 at the head instead: one call (quantMode -1) routes the rows and carries
+the per-token scales along as expandedScale, and emits the int64 cumsum (expertTokensNumType 0); scatter-type index
+(rowIdxType 1).
 ``fused_combine=True`` replaces the last two operators by aclnnGroupedMatmulFinalizeRoutingV3 (down projection with
 the weighted combine as scatter-add): routing then emits the gather-type index (rowIdxType 0), from which the glue
 derives the fused operator's rowIndex (destination token = source // K) and logit (the top-k weight of that source);
@@ -33,7 +35,7 @@ class MoeFfnW8A8:
     The operators see the reference layout [E, K, N] through transposed views of this storage.
     """
 
-    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v3", fused_combine=False,
+    def __init__(self, w13, w13_scale, w2, w2_scale, out_dtype=torch.bfloat16, routing="v2", fused_combine=False,
                  weight_nz=False, weight_row_major=False):
         assert routing in ("v2", "v3")
         assert not (fused_combine and routing != "v3")

@@ -39,11 +39,13 @@ def make_routing(cfg, seed=0):
     rng = np.random.default_rng(seed)
     logits = rng.standard_normal((cfg.tokens, cfg.experts), dtype=np.float32)
     if cfg.skew > 0:
-        # expert popularity ~ rank^-alpha (Zipf): bias = -alpha * log(rank), scaled so that the tail really empties
+        # expert popularity ~ rank^-alpha (Zipf): bias = -alpha * log(rank) on a random ranking of the experts.  With
+        # alpha = 1.2, 8192 tokens and top-8 of 256 this leaves 35-40 % of the experts without a row, about thirty
+        # experts with more than the mean of 256 rows and the most popular one with nearly every token (31 x the mean).
         perm = rng.permutation(cfg.experts)
         rank = np.empty(cfg.experts, np.float32)
         rank[perm] = np.arange(1, cfg.experts + 1, dtype=np.float32)
-        logits = logits + (-cfg.skew * 2.0 * np.log(rank))[None, :].astype(np.float32)
+        logits = logits + (-cfg.skew * np.log(rank))[None, :].astype(np.float32)
     z = logits - logits.max(axis=1, keepdims=True)
     p = np.exp(z)
     p /= p.sum(axis=1, keepdims=True)

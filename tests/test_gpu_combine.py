@@ -107,7 +107,7 @@ def test_fused_chain_matches_unfused_chain(pkg, dev):
     w13, w13s, w2, w2s = pkg.synth.make_weights(cfg, dev, seed=0)
     t = lambda a: torch.from_numpy(a).to(dev)
     plain = pkg.MoeFfnW8A8(w13, w13s, w2, w2s).forward(t(xq), t(xs), t(idx), t(wgt)).float().clone()
-    fused = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, fused_combine=True).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
+    fused = pkg.MoeFfnW8A8(w13, w13s, w2, w2s, routing="v3", fused_combine=True).forward(t(xq), t(xs), t(idx), t(wgt)).clone()
     torch.cuda.synchronize()
     assert fused.dtype == torch.float32
     err = (fused - plain).abs().max().item()

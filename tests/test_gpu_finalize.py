@@ -114,3 +114,50 @@ def test_no_scales_plain_gather(aclnn, dev):
     got = aclnn.moe_finalize_routing_v2(ex, idx, drop_pad_mode=0)
     torch.cuda.synchronize()
     assert torch.equal(got, ex[idx.long()])
+
+
+def _to_dtype(oracle, dtype, dev):
+    """(encode numpy fp32 -> oracle representation, oracle representation -> device tensor, oracle dtype code)."""
+    if dtype == "bf16":
+        enc = lambda a: None if a is None else oracle.f32_to_bf16_bits(a)
+        return enc, (lambda b: None if b is None else _bits_to_torch(b, dev)), oracle.DT_BF16
+    if dtype == "f16":
+        enc = lambda a: None if a is None else a.astype(np.float16).view(np.uint16)
+        return enc, (lambda b: None if b is None else torch.from_numpy(b.view(np.float16)).to(dev)), oracle.DT_F16
+    enc = lambda a: None if a is None else a
+    return enc, (lambda b: None if b is None else torch.from_numpy(b).to(dev)), oracle.DT_F32
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("K", [1, 3, 8])
+@pytest.mark.parametrize("seeds", ["none", "x1", "x1x2"])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_wide_rows_without_bias(aclnn, oracle, dev, dtype, K, seeds, mode):
+    """Rows of 1024 and more elements with no bias and at most eight experts per token take the batched kernel (indices
+    and weights loaded up front, row packets in pairs): its branches for dropped rows (index -1 in the drop/pad
+    arrangements, with the first term, a middle term or every term of a token dropped), for the x1 / x2 seeds without a
+    bias, and for fewer than eight experts per token in both index arrangements."""
+    rng = np.random.default_rng(1000 * mode + 10 * K + len(seeds))
+    T, H, E, C = 37, 1536, 5, 19
+    ex, idx, x1, x2, _, scales, _ = _case(rng, T, K, H, E, seeds != "none", seeds == "x1x2", False, mode, C)
+    if mode in (1, 3):
+        at = (lambda n, k: k * T + n) if mode == 1 else (lambda n, k: n * K + k)
+        idx[at(0, 0)] = -1                       # token 0: first term dropped
+        for k in range(K):
+            idx[at(1, k)] = -1                   # token 1: every term dropped
+        idx[at(2, K - 1)] = -1                   # token 2: last term dropped
+        if K >= 3:
+            idx[at(3, 0)] = 5                    # token 3: a middle term dropped, neighbours kept
+            idx[at(3, 1)] = -1
+            idx[at(3, 2)] = 7
+    enc, to_dev, code = _to_dtype(oracle, dtype, dev)
+    s_code = code
+    ref = oracle.moe_finalize_routing_v2(enc(ex), idx, enc(x1), enc(x2), None, enc(scales), None, drop_pad_mode=mode,
+                                         dtype=code, scale_dtype=s_code)
+    got = aclnn.moe_finalize_routing_v2(to_dev(enc(ex)), torch.from_numpy(idx).to(dev), to_dev(enc(x1)), to_dev(enc(x2)),
+                                        None, to_dev(enc(scales)), None, drop_pad_mode=mode)
+    torch.cuda.synchronize()
+    got_np = got.cpu().numpy() if dtype == "f32" else got.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got_np, ref)
+    if mode in (1, 3) and seeds == "none":
+        assert (got.float().cpu().numpy()[1] == 0).all()     # every term dropped and no seed: zeros

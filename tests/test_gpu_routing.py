@@ -49,7 +49,7 @@ def test_skewed_routing_bit_exact(pkg, aclnn, oracle, dev):
     cfg = pkg.synth.config(4)
     idx, _ = pkg.synth.make_routing(cfg, seed=4)
     hist = np.bincount(idx.reshape(-1), minlength=cfg.experts)
-    assert (hist == 0).mean() > 0.2 and hist.max() > 10 * hist.mean()
+    assert 0.25 <= (hist == 0).mean() <= 0.45 and hist.max() > 10 * hist.mean()   # the benchmark's ~30 % empty experts
     x = np.arange(cfg.tokens * 16, dtype=np.int32).reshape(cfg.tokens, 16).view(np.float32)
     for flag in (1, 2):
         ex, ri, cnt, _ = _run(aclnn, dev, x, idx, expert_num=cfg.experts, expert_tokens_count_or_cumsum_flag=flag)
