@@ -61,6 +61,7 @@ struct Plan {
     int64_t maxTiles = 0;   // launch bound on workgroups
     int32_t maxMTiles = 0;  // upper bound on m-tiles over all groups (M / tileM + groups)
     int32_t tilesN = 0;
+    bool pullTiles = false; // LDS-ring kernels: workgroups draw their tiles from counters instead of walking fixed shares
     uint64_t offSched = 0, offRowMax = 0, offS = 0;
     uint64_t workspaceBytes = 0;
 };

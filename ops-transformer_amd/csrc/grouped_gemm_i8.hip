@@ -56,10 +56,25 @@ constexpr int kMaxGroups = 1024;
 constexpr int kLdsBudget = 160 * 1024;
 
 // ---------------------------------------------------------------------------------------------- scheduling table
-// int32 layout: [0] total rows covered by groups, [1] total m-tiles, [2..2+G) row start, [..+G) rows, [..+G+1) m-tile prefix,
-// then one entry per m-tile (at most maxMTiles of them): the group it belongs to, so that the GEMM kernels find a
-// tile's group with one load instead of a binary search of dependent loads
-__host__ __device__ inline int SchedInts(int groups, int maxMTiles) { return 2 + 3 * groups + 1 + maxMTiles; }
+// int32 layout, all written by the scheduling kernel:
+//   header, 32 ints: [0] big m-tiles, [1] small m-tiles, [2] cost of the small ones, [3] cost of the big ones (see below),
+//                    [4] / [5] band width of the big / small run, [6] total rows covered by the groups;
+//   16 tile counters in one 128-byte line (32 ints): counter [2 * xcd + list], zeroed;
+//   the m-tile table, 4 ints per m-tile {group, first row, rows, 0} (at most maxMTiles of them): the big m-tiles in group
+//   order, then the small ones.  A GEMM kernel finds everything about a tile with one 16-byte load.
+// An m-tile is small when it holds at most kSmallRows rows: its time is the weight stream's (the whole K x 256 weight
+// block for a handful of rows), not the matrix pipe's.  The two kinds are kept apart so that a launch which holds both
+// (a skewed routing: a few experts with thousands of rows, many with a few) can run them side by side -- some
+// workgroups streaming small tiles while the others multiply big ones -- instead of a compute-bound phase followed by
+// a bandwidth-bound one.  Costs are in units of one 32-row MFMA tile over the whole K: a big m-tile costs its count of
+// occupied 32-row tiles (at least kSmallCost), a small one kSmallCost (what the weight stream of a tile takes when
+// only a part of the workgroups stream).
+constexpr int kSmallRows = 64;
+constexpr int kSmallCost = 3;
+constexpr int kQueueHeaderInts = 32;
+constexpr int kQueueCounterInts = 32;
+constexpr int kHdrCoveredRows = 6;
+__host__ __device__ inline int SchedTotalInts(int maxMTiles) { return kQueueHeaderInts + kQueueCounterInts + 4 * maxMTiles; }
 
 struct SchedArgs {
     const void* groupList;
@@ -93,6 +108,22 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
         __syncthreads();
         int32_t base = 0;
         for (int i = 0; i < wave; ++i) base += waveTotal[i];
+        return v + base;
+    };
+    // the same over two 32-bit counts packed into one 64-bit value (neither half may overflow into the other)
+    __shared__ uint64_t waveTotal64[16];
+    auto inclusiveScan64 = [&](uint64_t v) -> uint64_t {
+        const int lane = t & 63, wave = t >> 6;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint64_t below = __shfl_up(v, d, 64);
+            if (lane >= d) v += below;
+        }
+        __syncthreads();
+        if (lane == 63) waveTotal64[wave] = v;
+        __syncthreads();
+        uint64_t base = 0;
+        for (int i = 0; i < wave; ++i) base += waveTotal64[i];
         return v + base;
     };
     // group boundaries, clamped into [0, M] and made monotonic so that a malformed list cannot push rows out of range
@@ -146,7 +177,22 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
     end = end < begin ? begin : (end > a.M ? a.M : end);
     const int32_t rows = t < a.groups ? static_cast<int32_t>(end - begin) : 0;
     const int32_t tiles = (rows + a.tileM - 1) / a.tileM;
-    const int32_t tileInc = inclusiveScan(tiles);
+    // big and small m-tiles of this group (with tiles of at most kSmallRows rows every m-tile is small; otherwise only
+    // a group's last, partly filled m-tile can be) and the cost of the big ones; two packed prefix sums give every
+    // group the positions of its m-tiles in the two runs of the table, and the launch the totals
+    const bool allSmall = a.tileM <= kSmallRows;
+    const int32_t lastRows = tiles > 0 ? rows - (tiles - 1) * a.tileM : 0;
+    const int32_t smallCount = allSmall ? tiles : (tiles > 0 && lastRows <= kSmallRows ? 1 : 0);
+    const int32_t bigCount = tiles - smallCount;
+    int32_t bigCost = 0;
+    if (bigCount > 0) {
+        const bool lastIsBig = smallCount == 0;
+        const int32_t lastSub = (lastRows + 31) >> 5;
+        bigCost = (bigCount - (lastIsBig ? 1 : 0)) * max(a.tileM >> 5, kSmallCost) + (lastIsBig ? max(lastSub, kSmallCost) : 0);
+    }
+    const uint64_t countsInc = inclusiveScan64(static_cast<uint64_t>(tiles) | (static_cast<uint64_t>(bigCount) << 32));
+    const uint64_t costInc = inclusiveScan64(static_cast<uint64_t>(bigCost) | (static_cast<uint64_t>(tiles > 0 ? 1 : 0) << 32));
+    const int32_t tileInc = static_cast<int32_t>(countsInc & 0xffffffffu), bigInc = static_cast<int32_t>(countsInc >> 32);
     // rows covered by the list: the end of the last group, or with a sparse list the furthest end of any expert
     int32_t covered = static_cast<int32_t>(end);
     if (a.isCount == 2) {
@@ -159,34 +205,52 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
         covered = scan[0];
         __syncthreads();
     }
-    int32_t* rowStart = a.sched + 2;
-    int32_t* rowCount = rowStart + a.groups;
-    int32_t* tilePrefix = rowCount + a.groups;
-    if (t < a.groups) {
-        rowStart[t] = static_cast<int32_t>(begin);
-        rowCount[t] = rows;
-        tilePrefix[t] = tileInc - tiles;
-        if (t == a.groups - 1) {
-            tilePrefix[a.groups] = tileInc;
-            a.sched[0] = covered;
-            // A well-formed list never needs more than maxMTiles m-tiles (M / tileM + groups).  A malformed one whose
-            // groups overlap could: the tiles beyond the table are dropped, so no kernel indexes past it.
-            a.sched[1] = tileInc < a.maxMTiles ? tileInc : a.maxMTiles;
-        }
+    __shared__ int32_t sRowStart[kMaxGroups], sRows[kMaxGroups], sBigBefore[kMaxGroups], sSmallBefore[kMaxGroups];
+    __shared__ int32_t totals[4];
+    sRowStart[t] = static_cast<int32_t>(begin);
+    sRows[t] = rows;
+    sBigBefore[t] = bigInc - bigCount;
+    sSmallBefore[t] = (tileInc - bigInc) - smallCount;
+    __shared__ int32_t sCovered;
+    if (t == a.groups - 1) sCovered = covered;
+    if (t == 1023) {
+        totals[0] = bigInc;
+        totals[1] = tileInc - bigInc;
+        totals[2] = static_cast<int32_t>(costInc & 0xffffffffu);
+        totals[3] = static_cast<int32_t>(costInc >> 32);  // groups with rows
     }
     // group of every m-tile: scan[] takes the inclusive m-tile prefix (zero-tile groups repeat their
     // predecessor's value); m-tile m belongs to the first group whose inclusive prefix exceeds m
     scan[t] = t < a.groups ? tileInc : 0x7fffffff;
     __syncthreads();
     const int32_t totalMTiles = scan[a.groups - 1];
-    int32_t* const groupOfMTile = tilePrefix + a.groups + 1;
-    for (int32_t m = t; m < totalMTiles && m < a.maxMTiles; m += 1024) {
+    // A well-formed list never needs more than maxMTiles m-tiles (M / tileM + groups).  A malformed one whose groups
+    // overlap could: the m-tiles beyond the table are dropped, so no kernel indexes past it.
+    const int32_t nBig = min(totals[0], a.maxMTiles);
+    const int32_t nSmall = min(totals[1], a.maxMTiles - nBig);
+    if (t < kQueueCounterInts) a.sched[kQueueHeaderInts + t] = 0;
+    // Band width: with two or more m-tiles per group on average, four neighbouring m-tiles (mostly of one group) walk
+    // the n-tiles together and share each weight column block through L2; with one m-tile per group the n-tiles of a
+    // group follow each other, so that its activation rows are what stays in L2.  A small m-tile is its group's only
+    // one of its kind unless every tile is small.
+    const int32_t wideBands = totalMTiles >= 2 * totals[3] ? kGroupM : 1;
+    if (t < kQueueHeaderInts) {
+        a.sched[t] = t == 0 ? nBig : t == 1 ? nSmall : t == 2 ? nSmall * kSmallCost : t == 3 ? totals[2] : t == 4 ? wideBands
+                   : t == 5 ? (allSmall ? wideBands : 1) : t == kHdrCoveredRows ? sCovered : 0;
+    }
+    int4* const mTileTable = reinterpret_cast<int4*>(a.sched + kQueueHeaderInts + kQueueCounterInts);
+    for (int32_t m = t; m < totalMTiles; m += 1024) {
         int lo = -1, hi = a.groups - 1;  // scan[hi] > m always holds, scan[lo] <= m (lo = -1: nothing before)
         while (hi - lo > 1) {
             const int mid = (lo + hi) >> 1;
             if (scan[mid] > m) hi = mid; else lo = mid;
         }
-        groupOfMTile[m] = hi;
+        const int32_t inGroup = m - (hi > 0 ? scan[hi - 1] : 0);
+        const int32_t tileRows = min(a.tileM, sRows[hi] - inGroup * a.tileM);
+        const bool small = allSmall || tileRows <= kSmallRows;
+        const int32_t pos = small ? nBig + sSmallBefore[hi] + (allSmall ? inGroup : 0) : sBigBefore[hi] + inGroup;
+        const int32_t limit = small ? nBig + nSmall : nBig;
+        if (pos < limit) mTileTable[pos] = make_int4(hi, sRowStart[hi] + inGroup * a.tileM, tileRows, 0);
     }
 }
 
@@ -219,6 +283,11 @@ struct KernelArgs {
     // workgroup spans (include/opapi_profile.h): per workgroup {start, end} of the 100 MHz real-time counter and the
     // number of tiles it computed; null unless span recording is on
     uint64_t* wgSpans;
+    // LDS-ring kernels: the tile counters of the scheduling table as a pointer the kernel may write through (the table
+    // itself is a read-only kernel parameter), and whether workgroups pull their tiles from the counters (1) or walk a
+    // fixed share (0)
+    int32_t* queueCounters;
+    int32_t pullTiles;
 };
 
 // One output tile of one group, decoded from the scheduling table (all fields are wave-uniform).
@@ -231,33 +300,83 @@ struct TileInfo {
     int32_t colBase;  // first output channel (kSwiglu: first column of S)
 };
 
-// Position `local` of the XCD share that starts at logical tile `xcdFirst`.
-// `sched` is passed to the kernels as a __restrict__ parameter of its own: nothing in a GEMM kernel writes the table,
-// and telling the compiler so keeps these wave-uniform lookups on the scalar unit even after the kernel's stores.
+// Tile `logical` of one run of the m-tile table (`count` m-tiles from entry `first` on).  Bands of bandWidth m-tiles walk
+// the n-tiles together: consecutive tiles are the band's m-tiles at one n-tile, then the next n-tile.
 template <int kTileM, bool kSwiglu>
-__device__ __forceinline__ TileInfo DecodeTile(const KernelArgs& a, const int32_t* __restrict__ sched, int64_t xcdFirst,
-                                               int64_t perXcd, int64_t totalTiles, int64_t local) {
+__device__ __forceinline__ TileInfo DecodeListTile(const KernelArgs& a, const int4* __restrict__ table, int32_t first,
+                                                   int32_t count, int32_t bandWidth, int64_t logical) {
     TileInfo t{};
-    const int64_t logical = xcdFirst + local;
-    if (local >= perXcd || logical >= totalTiles) return t;
-    const int32_t* const rowStartTbl = sched + 2;
-    const int32_t* const rowCountTbl = rowStartTbl + a.groups;
-    const int32_t* const tilePrefix = rowCountTbl + a.groups;
-    const int32_t q = static_cast<int32_t>(logical / a.tilesN);
-    const int lo = tilePrefix[a.groups + 1 + q];  // group of m-tile q
-    const int32_t inGroup = static_cast<int32_t>(logical - static_cast<int64_t>(tilePrefix[lo]) * a.tilesN);
-    const int32_t tilesM = tilePrefix[lo + 1] - tilePrefix[lo];
-    const int32_t band = inGroup / (kGroupM * a.tilesN);
-    const int32_t rem = inGroup % (kGroupM * a.tilesN);
-    const int32_t bandTiles = min(kGroupM, tilesM - kGroupM * band);
-    const int32_t tileMIdx = kGroupM * band + rem % bandTiles;
+    const int32_t perBand = bandWidth * a.tilesN;
+    const int32_t band = static_cast<int32_t>(logical / perBand);
+    const int32_t rem = static_cast<int32_t>(logical % perBand);
+    const int32_t bandTiles = min(bandWidth, count - bandWidth * band);
+    const int4 e = table[first + bandWidth * band + rem % bandTiles];
     t.valid = 1;
-    t.group = lo;
+    t.group = e.x;
+    t.rowBase = e.y;
+    t.rows = e.z;  // 1..kTileM
     t.tileN = rem / bandTiles;
-    t.rowBase = rowStartTbl[lo] + tileMIdx * kTileM;
-    t.rows = min(kTileM, rowCountTbl[lo] - tileMIdx * kTileM);  // >= 1
     t.colBase = kSwiglu ? t.tileN * (kTileN / 2) : t.tileN * kTileN;
     return t;
+}
+
+// ---- tile counters: workgroups pull their tiles instead of walking a fixed share ----
+// Each of the two runs of the m-tile table (big, small) is cut into eight contiguous shares of tiles, one per XCD, so
+// that the workgroups of an XCD sit on neighbouring tiles and share operands through that XCD's L2.  Counter
+// [2 * xcd + list] hands out the tiles of a share in order.  A workgroup draws from its own XCD first -- the list it
+// prefers, then the other -- and, when both are used up, from the other XCDs' shares in ring order, so nobody idles
+// while tiles are left anywhere.  The counters are only ever added to (values past a share's size mean "used up").
+// (The lists' sizes travel as plain values: a structure handed round by reference, or an array indexed at run time,
+// ends up in scratch memory.)
+__device__ __forceinline__ void QueueShare(int64_t tilesBig, int64_t tilesSmall, int counter, int64_t* first, int64_t* size) {
+    const int64_t total = (counter & 1) ? tilesSmall : tilesBig;
+    const int64_t per = (total + kXcds - 1) / kXcds;
+    const int64_t begin = (counter >> 1) * per;
+    *first = begin;
+    *size = total - begin < 0 ? 0 : (total - begin < per ? total - begin : per);
+}
+// Counter i-th in the preference order of a workgroup on XCD `home` that prefers list `prefer`.
+__device__ __forceinline__ int QueueCandidate(int i, int home, int prefer) {
+    return 2 * ((home + (i >> 1)) & (kXcds - 1)) + ((i & 1) ? 1 - prefer : prefer);
+}
+__device__ __forceinline__ int QueueFirstOpen(uint32_t usedUp, int home, int prefer) {
+#pragma unroll
+    for (int i = 0; i < 2 * kXcds; ++i) {
+        const int c = QueueCandidate(i, home, prefer);
+        if (((usedUp >> c) & 1u) == 0) return c;
+    }
+    return -1;
+}
+__device__ __forceinline__ int32_t QueueTake(int32_t* counters, int c) {
+    return __hip_atomic_fetch_add(counters + c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Completes a draw that began with QueueTake on counter c (value v; c < 0: nothing was open): returns the list (0 big,
+// 1 small) and the tile inside that list's run, or list -1 when every share is used up.  One thread of the workgroup.
+struct QueueDraw {
+    int32_t list;     // 0 big, 1 small, -1 none
+    int32_t logical;  // tile inside that list's run
+    uint32_t usedUp;  // the caller's mask of used-up counters, updated
+};
+__device__ __forceinline__ QueueDraw QueueResolve(int64_t tilesBig, int64_t tilesSmall, int32_t* counters, int home, int prefer,
+                                                  uint32_t usedUp, int c, int32_t v) {
+    while (c >= 0) {
+        int64_t first, size;
+        QueueShare(tilesBig, tilesSmall, c, &first, &size);
+        if (v < size) return QueueDraw{c & 1, static_cast<int32_t>(first + v), usedUp};
+        usedUp |= 1u << c;
+        // a look at all sixteen counters at once (one round trip) spares a failed draw, i.e. a round trip, per used-up share
+        int32_t now[2 * kXcds];  // fully unrolled below: stays in registers
+#pragma unroll
+        for (int i = 0; i < 2 * kXcds; ++i) now[i] = __hip_atomic_load(counters + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int i = 0; i < 2 * kXcds; ++i) {
+            QueueShare(tilesBig, tilesSmall, i, &first, &size);
+            if (now[i] >= size) usedUp |= 1u << i;
+        }
+        c = QueueFirstOpen(usedUp, home, prefer);
+        if (c >= 0) v = QueueTake(counters, c);
+    }
+    return QueueDraw{-1, 0, usedUp};
 }
 
 // Output channel held in row r of the weight tile (clamped: channels past N are loaded but never stored).
@@ -295,10 +414,15 @@ __device__ __forceinline__ int64_t WeightRowBase(const KernelArgs& a, int32_t n)
 // owns column blocks ni = 0, 1, lane l32 inside each (plain: 64*waveN + 32*ni; kSwiglu: S column 32*waveN and its partner).
 // Only the first mySub accumulator tiles of the wave are real.  ldsRowScale holds the tile's per-row scales.
 // Contains workgroup barriers: every wave must call it.
-template <int kSubM, int kTileM, Epilogue kEpi>
+// afterScaleLoads() is called once the channel scales of the tile have been requested and before anything is stored: a
+// memory request made there queues behind loads whose answers the epilogue needs first, not in front of them.
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+template <int kSubM, int kTileM, Epilogue kEpi, typename Hook = NoHook>
 __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo& t, v16i (&acc)[kSubM][2], int mySub,
                                              int waveRow0, int waveN, int l32, int lhi, int tid,
-                                             const float* ldsRowScale, float* ldsRowMax) {
+                                             const float* ldsRowScale, float* ldsRowMax, Hook afterScaleLoads = NoHook{}) {
     const int32_t rows = t.rows, rowBase = t.rowBase, group = t.group;
     // The row / address arithmetic below depends only on the lane; hoisted out of the persistent tile loop it would
     // stay alive across the whole kernel and spill, and a reload in here waits for every store issued so far.  An
@@ -321,6 +445,7 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
             if (valid0) bias0 = LoadScale(a.bias, static_cast<int64_t>(group) * a.N + n0, a.biasDtype);
             if (valid1) bias1 = LoadScale(a.bias, static_cast<int64_t>(group) * a.N + n0 + 32, a.biasDtype);
         }
+        afterScaleLoads();
         // 16-bit outputs: a lane holds one column of each block, i.e. 2-byte pieces 64 bytes apart.  Neighbouring lanes
         // swap one value so that an even lane owns columns (c, c+1) of block 0 and the odd lane next to it the same pair
         // of block 1; every lane then stores one aligned 32-bit word and a half-wave covers a whole 128-byte row segment.
@@ -461,6 +586,7 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
             scA = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + j, a.scaleDtype);
             scB = LoadScale(a.scale, static_cast<int64_t>(group) * a.N + a.halfN + j, a.scaleDtype);
         }
+        afterScaleLoads();
         const bool wholeColumns = t.colBase + 32 * waveN + 32 <= a.halfN;  // wave-uniform
 #pragma unroll
         for (int mi = 0; mi < kSubM; ++mi) {
@@ -603,7 +729,8 @@ struct StreamCfg {
     static constexpr int kTileM = 32 * (kSub0 + kSub1);
     static constexpr int kStageBytesA = kTileM * kStep;
     static constexpr int kStageBytesB = kTileN * kStep;
-    static constexpr int kScratchBytes = (1 + kWavesN) * kTileM * 4;
+    static constexpr int kQueueLdsInts = 16;  // the workgroup's tile sequence (four {list, tile} pairs) and its draw state
+    static constexpr int kScratchBytes = (1 + kWavesN) * kTileM * 4 + kQueueLdsInts * 4;
     static constexpr bool kStaggered = kTileM == 192;
     static constexpr int kFitWhole = (kLdsBudget - kScratchBytes) / (kStageBytesA + kStageBytesB);
     static constexpr int kStagesB = kStaggered ? (kLdsBudget - kScratchBytes - 2 * kStageBytesA) / kStageBytesB
@@ -729,16 +856,77 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     const int l32 = lane & 31;
     const int lhi = lane >> 5;
 
-    const int64_t totalTiles = static_cast<int64_t>(sched[1]) * a.tilesN;
+    // ---- this workgroup's sequence of tiles ----
+    // Workgroup b serves XCD b % 8 as its slot b / 8.  With a.pullTiles the sequence comes out of the tile counters (see
+    // QueueShare): thread 0 draws, the result reaches the other waves through a four-entry ring in LDS, and tile n + 2
+    // is drawn while tile n's epilogue runs (the draw goes out at its head, the answer is looked at behind it),
+    // because the issue side already reads tile n + 1's operands during tile n.  Otherwise the two runs of
+    // the m-tile table are one list cut into eight fixed shares, which the workgroups of an XCD walk with stride
+    // gridDim / 8.
+    const int32_t* const queueHdr = sched;
+    const int32_t countBig = queueHdr[0], countSmall = queueHdr[1];  // m-tiles per list
+    const int32_t bandBig = queueHdr[4], bandSmall = queueHdr[5];
+    const int4* const mTileTable = reinterpret_cast<const int4*>(queueHdr + kQueueHeaderInts + kQueueCounterInts);
+    const int xcd = blockIdx.x % kXcds;
+    const int32_t slots = gridDim.x / kXcds;
+    const int32_t slot = blockIdx.x / kXcds;
+    const bool pull = a.pullTiles != 0;
+    const int64_t bigTiles = static_cast<int64_t>(countBig) * a.tilesN;
+    const int64_t totalTiles = bigTiles + static_cast<int64_t>(countSmall) * a.tilesN;
     const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
-    const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
-    const int64_t slots = gridDim.x / kXcds;
-    auto decode = [&](int64_t local) __attribute__((always_inline)) { return DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, local); };
+    const int64_t xcdFirst = static_cast<int64_t>(xcd) * perXcd;
+    int32_t* const ldsSeq = reinterpret_cast<int32_t*>(ldsRowMax + kWavesN * kTileM);
+    constexpr int kSeqUsedUp = 8, kSeqDrawCounter = 9;  // thread 0's draw state, behind the ring
+    // Which list this workgroup draws from first: the small m-tiles get the share of each XCD's workgroups that their
+    // cost is of the whole, so that both lists run dry at about the same time; until then a part of the machine
+    // streams weights for a handful of rows each while the rest multiplies.
+    int prefer = 0;
+    {
+        const int64_t costSmall = queueHdr[2], costAll = costSmall + queueHdr[3];
+        int64_t forSmall = costAll > 0 ? (slots * costSmall + costAll / 2) / costAll : 0;
+        if (forSmall == 0 && countSmall > 0 && slots > 1) forSmall = 1;
+        if (countBig == 0) forSmall = slots;
+        prefer = slot < forSmall ? 1 : 0;
+    }
+    auto listTile = [&](int32_t list, int64_t logical) __attribute__((always_inline)) {
+        return DecodeListTile<kTileM, kSwiglu>(a, mTileTable, list ? countBig : 0, list ? countSmall : countBig,
+                                               list ? bandSmall : bandBig, logical);
+    };
+    // the n-th tile of this workgroup (n at most two ahead of the tile being computed)
+    auto tileAt = [&](int32_t n) __attribute__((always_inline)) -> TileInfo {
+        if (pull) {
+            const int32_t list = __builtin_amdgcn_readfirstlane(ldsSeq[2 * (n & 3)]);
+            const int32_t logical = __builtin_amdgcn_readfirstlane(ldsSeq[2 * (n & 3) + 1]);
+            if (list < 0) return TileInfo{};
+            return listTile(list, logical);
+        }
+        const int64_t local = slot + static_cast<int64_t>(n) * slots;
+        const int64_t logical = xcdFirst + local;
+        if (local >= perXcd || logical >= totalTiles) return TileInfo{};
+        return logical < bigTiles ? listTile(0, logical) : listTile(1, logical - bigTiles);
+    };
+    if (pull) {
+        if (tid == 0) {
+            // the first two tiles: both draws go out together
+            uint32_t usedUp = 0;
+            const int c = QueueFirstOpen(usedUp, xcd, prefer);
+            const int32_t v0 = QueueTake(a.queueCounters, c);
+            const int32_t v1 = QueueTake(a.queueCounters, c);
+            QueueDraw d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer, usedUp, c, v0);
+            ldsSeq[0] = d.list;
+            ldsSeq[1] = d.logical;
+            if (d.list >= 0) d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer, d.usedUp, c, v1);
+            ldsSeq[2] = d.list;
+            ldsSeq[3] = d.logical;
+            ldsSeq[kSeqUsedUp] = static_cast<int32_t>(d.usedUp);
+        }
+        __syncthreads();
+    }
 
     const uint64_t spanStart = a.wgSpans != nullptr ? __builtin_amdgcn_s_memrealtime() : 0;
     uint64_t spanTiles = 0;
-    int64_t local = blockIdx.x / kXcds;
-    TileInfo cur = decode(local);
+    int32_t curNo = 0;  // position of the tile being computed in this workgroup's sequence
+    TileInfo cur = tileAt(0);
     if (!cur.valid) {
         if (a.wgSpans != nullptr && tid == 0) {
             a.wgSpans[3 * blockIdx.x] = spanStart;
@@ -758,7 +946,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     // (Plain variables, picked by if constexpr: a cursor struct handed round by reference ends up in vector registers.)
     const uint32_t ldsBase = LdsAddress(lds);
     TileInfo issTileA = cur, issTileB = cur;
-    int64_t issLocalA = local, issLocalB = local;
+    int32_t issNoA = 0, issNoB = 0;            // position of each cursor's tile in the sequence
     int issStepA = 0, issStepB = 0;            // k-step of the tile that goes out next
     int issSlotA = 0, issSlotB = 0;            // ring buffer it goes into
     bool issDrainedA = false, issDrainedB = false;  // no further tile: the issue slots re-read one hot kilobyte (see advance)
@@ -826,7 +1014,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         constexpr int kParts = decltype(partsTag)::value;
         constexpr bool kCursorA = kParts == kPartA;
         TileInfo& tile = kCursorA ? issTileA : issTileB;
-        int64_t& tileLocal = kCursorA ? issLocalA : issLocalB;
+        int32_t& tileNo = kCursorA ? issNoA : issNoB;
         int& step = kCursorA ? issStepA : issStepB;
         int& slot = kCursorA ? issSlotA : issSlotB;
         bool& drained = kCursorA ? issDrainedA : issDrainedB;
@@ -838,10 +1026,10 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             // every one of them then re-reads the same first kilobyte of the last tile's weights, which stays in L2,
             // instead of pulling more stages of weights from HBM per workgroup.
             step = 0;
-            const TileInfo next = decode(tileLocal + slots);
+            const TileInfo next = tileAt(tileNo + 1);
             if (next.valid) {
                 tile = next;
-                tileLocal += slots;
+                ++tileNo;
                 setupIssue(tile, partsTag);
             } else if (!drained) {
                 drained = true;
@@ -959,7 +1147,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     v16i acc[kSubM][2];
 
     while (true) {
-        const TileInfo following = decode(local + slots);
+        const TileInfo following = tileAt(curNo + 1);
         // the next tile's per-row scale travels in a register until this tile's epilogue has read the LDS copy
         float followingRowScale = 0.0f;
         if (following.valid && kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
@@ -1085,16 +1273,35 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
         }
         ForCount<kSub0>(mySub, runTile);
 
-        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, waveN, Opaque(l32), Opaque(lhi), Opaque(tid), ldsRowScale, ldsRowMax);
+        // The draw for the tile after the next goes out inside the epilogue and is looked at behind it.  A wave's memory
+        // requests are counted back in issue order and the draw, an atomic that is settled at the memory side, takes
+        // microseconds on a loaded machine: in front of the k loop it would hold up the count of every operand stage
+        // issued after it.  During the epilogue the ring is full and nothing is issued.
+        int32_t drawValue = 0;
+        auto draw = [&]() __attribute__((always_inline)) {
+            if (pull && following.valid && tid == 0) {
+                const int c = QueueFirstOpen(static_cast<uint32_t>(ldsSeq[kSeqUsedUp]), xcd, prefer);
+                ldsSeq[kSeqDrawCounter] = c;
+                if (c >= 0) drawValue = QueueTake(a.queueCounters, c);
+            }
+        };
+        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, waveN, Opaque(l32), Opaque(lhi), Opaque(tid), ldsRowScale, ldsRowMax, draw);
         // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
         // stores and the DMAs in flight, which had the whole epilogue to land) before counting DMAs again.
         WaitVmcnt<0>();
         ++spanTiles;
         if (!following.valid) break;
-        __syncthreads();  // the epilogue's reads of ldsRowScale / ldsRowMax are done
+        if (pull && tid == 0) {
+            const QueueDraw d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer,
+                                             static_cast<uint32_t>(ldsSeq[kSeqUsedUp]), ldsSeq[kSeqDrawCounter], drawValue);
+            ldsSeq[2 * ((curNo + 2) & 3)] = d.list;
+            ldsSeq[2 * ((curNo + 2) & 3) + 1] = d.logical;
+            ldsSeq[kSeqUsedUp] = static_cast<int32_t>(d.usedUp);
+        }
+        __syncthreads();  // the epilogue's reads of ldsRowScale / ldsRowMax are done; the drawn tile is in the ring
         if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) ldsRowScale[tid] = followingRowScale;
         cur = following;
-        local += slots;
+        ++curNo;
     }
     if (a.wgSpans != nullptr && tid == 0) {
         a.wgSpans[3 * blockIdx.x] = spanStart;
@@ -1129,11 +1336,19 @@ __global__ __launch_bounds__(256) void GenericGemmKernel(KernelArgs a, const int
     const int l32 = lane & 31;
     const int lhi = lane >> 5;
 
-    const int64_t totalTiles = static_cast<int64_t>(sched[1]) * a.tilesN;
+    // one tile per workgroup: the two runs of the m-tile table as one list, cut into eight contiguous shares
+    const int32_t* const queueHdr = sched;
+    const int4* const mTileTable = reinterpret_cast<const int4*>(queueHdr + kQueueHeaderInts + kQueueCounterInts);
+    const int32_t countBig = queueHdr[0], countSmall = queueHdr[1];
+    const int64_t bigTiles = static_cast<int64_t>(countBig) * a.tilesN;
+    const int64_t totalTiles = bigTiles + static_cast<int64_t>(countSmall) * a.tilesN;
     const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
-    const int64_t xcdFirst = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd;
-    const TileInfo t = DecodeTile<kTileM, kSwiglu>(a, sched, xcdFirst, perXcd, totalTiles, blockIdx.x / kXcds);
-    if (!t.valid) return;
+    const int64_t local = blockIdx.x / kXcds;
+    const int64_t logical = static_cast<int64_t>(blockIdx.x % kXcds) * perXcd + local;
+    if (local >= perXcd || logical >= totalTiles) return;
+    const TileInfo t = logical < bigTiles
+        ? DecodeListTile<kTileM, kSwiglu>(a, mTileTable, 0, countBig, queueHdr[4], logical)
+        : DecodeListTile<kTileM, kSwiglu>(a, mTileTable, countBig, countSmall, queueHdr[5], logical - bigTiles);
     if (kEpi != Epilogue::kInt32 && a.rowScale != nullptr && tid < kTileM) {
         ldsRowScale[tid] = a.rowScale[t.rowBase + (tid < t.rows ? tid : t.rows - 1)];
     }
@@ -1217,7 +1432,7 @@ __device__ __forceinline__ int8_t QuantOne(float s, float inv) {
 // maxima for itself (a handful of L2 hits): the row's two dependent memory round trips overlap and there is no barrier.
 __global__ __launch_bounds__(256) void RequantKernel(RequantArgs a) {
     const int64_t row = blockIdx.x;
-    if (row >= a.sched[0]) return;
+    if (row >= a.sched[kHdrCoveredRows]) return;
     typedef float Float4 __attribute__((ext_vector_type(4)));
     const float* src = a.s + row * a.halfN;
     int8_t* dst = a.y + row * a.halfN;
@@ -1400,6 +1615,14 @@ Plan MakePlan(const Problem& p) {
     } else {
         plan.tileM = want <= 32.0 ? 32 : 128;
     }
+    // Workgroups pull their tiles from counters where a tile is long enough to hide the draw: at least eight k-steps
+    // (the issue side then never runs more than one tile ahead, which is what the two-tile look-ahead of the draw
+    // covers) and more than 64 rows; the handful-of-rows tiles of a decode step keep their fixed shares.
+    // OPAPI_GEMM_PULL=0 / 1 switches it off / on for every shape with eight k-steps.
+    plan.pullTiles = StreamOk(p) && p.K / 128 >= 8 && plan.tileM > 64 && plan.maxTiles < (1ll << 31);
+    if (const char* env = std::getenv("OPAPI_GEMM_PULL")) {
+        plan.pullTiles = StreamOk(p) && p.K / 128 >= 8 && plan.maxTiles < (1ll << 31) && std::atoi(env) != 0;
+    }
     plan.wavesM = plan.tileM >= 64 && StreamOk(p) ? 2 : 1;
     plan.subTilesM = (plan.tileM / 32 + plan.wavesM - 1) / plan.wavesM;
     const int64_t maxMTiles = p.M / plan.tileM + groups;
@@ -1408,7 +1631,7 @@ Plan MakePlan(const Problem& p) {
     plan.maxTiles = (maxMTiles * plan.tilesN + kXcds - 1) / kXcds * kXcds;
     uint64_t off = 0;
     plan.offSched = off;
-    off += Align256(static_cast<uint64_t>(SchedInts(static_cast<int>(groups), plan.maxMTiles)) * 4);
+    off += Align256(static_cast<uint64_t>(SchedTotalInts(plan.maxMTiles)) * 4);
     if (p.epilogue == Epilogue::kSwiglu) {
         plan.offRowMax = off;
         off += Align256(static_cast<uint64_t>(p.M) * 4 * static_cast<uint64_t>(plan.tilesN));
@@ -1472,6 +1695,8 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.bias = p.bias;
     ka.biasDtype = p.biasDtype;
     ka.wgSpans = nullptr;
+    ka.queueCounters = sched + kQueueHeaderInts;
+    ka.pullTiles = plan.pullTiles ? 1 : 0;
 
     hipError_t e = hipSuccess;
     if (p.K > 0) {

@@ -409,3 +409,65 @@ def test_many_tiles_per_workgroup_other_layouts(aclnn, oracle, dev, monkeypatch,
     assert np.array_equal(acc.cpu().numpy(), oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True))
     ref = oracle.grouped_matmul_dequant(x, wt, scale, pt, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
     assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+
+
+@pytest.mark.parametrize("K", [1024, 1152])
+@pytest.mark.parametrize("tile_m", [32, 64, 96, 128, 160, 192, 256])
+def test_pulled_tiles_under_skew_every_height(aclnn, oracle, dev, monkeypatch, tile_m, K):
+    """Tiles of eight k-steps and more are drawn from the tile counters (forced on here for the two smallest heights as
+    well).  A skewed list -- two groups of many m-tiles, a few of a few hundred rows, many of a handful, some empty,
+    sizes either side of the small-tile limit of 64 rows and of each tile height -- fills both runs of the m-tile
+    table, gives every workgroup several tiles, and ends with workgroups drawing from other XCDs' shares.  K = 1024 is
+    the shortest tile that is pulled (the issue side reaches the tile after next exactly when it has been drawn).
+    int32 output bit-exact, and the down-projection epilogue on the same list."""
+    monkeypatch.setenv("OPAPI_GEMM_TILE_M", str(tile_m))
+    monkeypatch.setenv("OPAPI_GEMM_PULL", "1")
+    rng = np.random.default_rng(7 * tile_m + K)
+    N = 256 * 16 + 64
+    sizes = [1500, 3, 700, 0, 40, 300, 1, 65, 64, 513, 0, 63, tile_m, tile_m + 1, max(tile_m - 1, 1), 2 * tile_m]
+    sizes += [int(v) for v in rng.integers(1, 24, 30)]
+    sizes = np.array(sizes)
+    E = len(sizes)
+    cumsum = np.cumsum(sizes).astype(np.int64)
+    M = int(cumsum[-1])
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    wv = [_weight_views(wt, dev, "kmajor")]
+    acc = aclnn.grouped_matmul_v4([t(x)], wv, group_list=t(cumsum), split_item=3, group_type=0)[0]
+    y = aclnn.grouped_matmul_v4([t(x)], wv, scale=[t(scale)], per_token_scale=[t(pt)], group_list=t(sizes.astype(np.int64)),
+                                split_item=3, group_type=0, group_list_type=1, output_dtype=torch.bfloat16)[0]
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True))
+    ref = oracle.grouped_matmul_dequant(x, wt, scale, pt, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+    # the same launch with fixed shares gives the same bits
+    monkeypatch.setenv("OPAPI_GEMM_PULL", "0")
+    acc_fixed = aclnn.grouped_matmul_v4([t(x)], wv, group_list=t(cumsum), split_item=3, group_type=0)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(acc, acc_fixed)
+
+
+def test_pulled_tiles_swiglu_skewed(aclnn, oracle, dev, monkeypatch):
+    """The SwiGLU epilogue on a skewed list with pulled tiles (the requantisation reads rows written by tiles that ran
+    in no fixed order)."""
+    monkeypatch.setenv("OPAPI_GEMM_PULL", "1")
+    rng = np.random.default_rng(99)
+    K, N = 1024, 2048
+    sizes = np.array([900, 2, 0, 300, 17, 64, 65, 1, 5, 130, 40, 0, 7] + [int(v) for v in rng.integers(1, 12, 20)])
+    E = len(sizes)
+    cumsum = np.cumsum(sizes).astype(np.int64)
+    M = int(cumsum[-1])
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    q, qs = aclnn.grouped_matmul_swiglu_quant(t(x), _weight_views(wt, dev, "kmajor"), t(cumsum), t(scale), t(pt))
+    torch.cuda.synchronize()
+    q_ref, qs_ref = oracle.grouped_matmul_swiglu_quant(x, wt, scale, pt, cumsum, w_trans=True)
+    diff = np.abs(q.cpu().numpy().astype(np.int32) - q_ref.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+    np.testing.assert_allclose(qs.cpu().numpy(), qs_ref, rtol=1e-5)
