@@ -413,16 +413,21 @@ __device__ __forceinline__ int64_t WeightRowBase(const KernelArgs& a, int32_t n)
 // Epilogue of one tile.  acc[mi][ni][v] is C[row, col] with row = waveRow0 + 32*mi + 8*(v/4) + 4*lhi + (v%4); the wave
 // owns column blocks ni = 0, 1, lane l32 inside each (plain: 64*waveN + 32*ni; kSwiglu: S column 32*waveN and its partner).
 // Only the first mySub accumulator tiles of the wave are real.  ldsRowScale holds the tile's per-row scales.
-// Contains workgroup barriers: every wave must call it.
 // afterScaleLoads() is called once the channel scales of the tile have been requested and before anything is stored: a
 // memory request made there queues behind loads whose answers the epilogue needs first, not in front of them.
 struct NoHook {
     __device__ __forceinline__ void operator()() const {}
 };
-template <int kSubM, int kTileM, Epilogue kEpi, typename Hook = NoHook>
-__device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo& t, v16i (&acc)[kSubM][2], int mySub,
-                                             int waveRow0, int waveN, int l32, int lhi, int tid,
-                                             const float* ldsRowScale, float* ldsRowMax, Hook afterScaleLoads = NoHook{}) {
+//
+// A wave that holds kNi = 4 column blocks (four waves per tile, 128 x 128 each) calls the per-wave part once per pair
+// of blocks: kPair picks acc[mi][2 * kPair] and acc[mi][2 * kPair + 1], and waveN is then the column position
+// 0..3 that this pair has in the tile (what the wave index is when eight waves hold one pair each).
+template <int kSubM, int kNi, int kPair, int kTileM, Epilogue kEpi, typename Hook = NoHook>
+__device__ __forceinline__ void TileEpilogueWave(const KernelArgs& a, const TileInfo& t, v16i (&accAll)[kSubM][kNi], int mySub,
+                                                 int waveRow0, int waveN, int l32, int lhi,
+                                                 const float* ldsRowScale, float* ldsRowMax, Hook afterScaleLoads = NoHook{}) {
+    // the pair's two accumulator columns under the name the code below uses: acc(mi, 0 / 1)
+    auto acc = [&](int mi, int j) __attribute__((always_inline)) -> v16i& { return accAll[mi][2 * kPair + j]; };
     const int32_t rows = t.rows, rowBase = t.rowBase, group = t.group;
     // The row / address arithmetic below depends only on the lane; hoisted out of the persistent tile loop it would
     // stay alive across the whole kernel and spill, and a reload in here waits for every store issued so far.  An
@@ -484,8 +489,8 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int v = 4 * q + i;
-                        const Float2 f = {__fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), sc0), rsv[i]),
-                                          __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), sc1), rsv[i])};
+                        const Float2 f = {__fmul_rn(__fmul_rn(static_cast<float>(acc(mi, 0)[v]), sc0), rsv[i]),
+                                          __fmul_rn(__fmul_rn(static_cast<float>(acc(mi, 1)[v]), sc1), rsv[i])};
                         uint32_t pk;
                         if constexpr (kToBf16) {
                             pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));
@@ -524,12 +529,12 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                 const int r = waveRow0 + 32 * mi + 8 * (v / 4) + 4 * lhi + (v % 4);
                 const int64_t rowOff = static_cast<int64_t>(rowBase + r) * a.N;
                 if (kEpi == Epilogue::kInt32) {
-                    if (r < rows && valid0) static_cast<int32_t*>(a.out)[rowOff + n0] = acc[mi][0][v];
-                    if (r < rows && valid1) static_cast<int32_t*>(a.out)[rowOff + n0 + 32] = acc[mi][1][v];
+                    if (r < rows && valid0) static_cast<int32_t*>(a.out)[rowOff + n0] = acc(mi, 0)[v];
+                    if (r < rows && valid1) static_cast<int32_t*>(a.out)[rowOff + n0 + 32] = acc(mi, 1)[v];
                     continue;
                 }
-                float y0 = __fmul_rn(static_cast<float>(acc[mi][0][v]), sc0);
-                float y1 = __fmul_rn(static_cast<float>(acc[mi][1][v]), sc1);
+                float y0 = __fmul_rn(static_cast<float>(acc(mi, 0)[v]), sc0);
+                float y1 = __fmul_rn(static_cast<float>(acc(mi, 1)[v]), sc1);
                 if (hasRowScale) {
                     const float rs = ldsRowScale[r < rows ? r : 0];
                     y0 = __fmul_rn(y0, rs);
@@ -606,8 +611,8 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int v = 4 * q + i;
-                        const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), xsv[i]), scA);
-                        const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xsv[i]), scB);
+                        const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc(mi, 0)[v]), xsv[i]), scA);
+                        const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc(mi, 1)[v]), xsv[i]), scB);
                         float sv = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
                         const bool ok = kFull || rTop + 8 * q + 4 * lhi + i < rows;
                         if (ok) __builtin_nontemporal_store(sv, &sTile[static_cast<int64_t>(8 * q + i) * a.halfN + laneOff]);
@@ -668,8 +673,8 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                 float s = 0.0f;
                 if (valid) {
                     const float xs = ldsRowScale[r];
-                    const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][0][v]), xs), scA);
-                    const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc[mi][1][v]), xs), scB);
+                    const float ca = __fmul_rn(__fmul_rn(static_cast<float>(acc(mi, 0)[v]), xs), scA);
+                    const float cb = __fmul_rn(__fmul_rn(static_cast<float>(acc(mi, 1)[v]), xs), scB);
                     // swish(ca) * cb with the hardware exp2 / reciprocal: a few ulp from the correctly rounded value,
                     // far inside the +-1 LSB the int8 requantisation is held to
                     s = __fmul_rn(__fmul_rn(ca, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-ca)))), cb);
@@ -682,15 +687,31 @@ __device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo
                 if (l32 == 0) ldsRowMax[waveN * kTileM + r] = m;
             }
         }
-        __syncthreads();
-        // one partial maximum per (n-tile, row): no atomics and nothing to pre-zero; the requantisation folds them
-        if (tid < rows) {
-            float m = ldsRowMax[tid];
-#pragma unroll
-            for (int w = 1; w < kWavesN; ++w) m = fmaxf(m, ldsRowMax[w * kTileM + tid]);
-            a.rowMax[static_cast<int64_t>(t.tileN) * a.M + rowBase + tid] = m;
-        }
     }
+}
+
+// The part of the kSwiglu epilogue that follows the waves' own work: folds the four column positions' partial row maxima
+// into one per (n-tile, row).  Contains a workgroup barrier: every wave must call it (the workgroup has at least
+// kTileM threads).
+template <int kTileM>
+__device__ __forceinline__ void TileEpilogueFoldMax(const KernelArgs& a, const TileInfo& t, int tid, const float* ldsRowMax) {
+    __syncthreads();
+    // one partial maximum per (n-tile, row): no atomics and nothing to pre-zero; the requantisation folds them
+    if (tid < t.rows) {
+        float m = ldsRowMax[tid];
+#pragma unroll
+        for (int w = 1; w < kWavesN; ++w) m = fmaxf(m, ldsRowMax[w * kTileM + tid]);
+        a.rowMax[static_cast<int64_t>(t.tileN) * a.M + t.rowBase + tid] = m;
+    }
+}
+
+// Eight-wave form (one pair of column blocks per wave): the per-wave part, then the fold.
+template <int kSubM, int kTileM, Epilogue kEpi, typename Hook = NoHook>
+__device__ __forceinline__ void TileEpilogue(const KernelArgs& a, const TileInfo& t, v16i (&acc)[kSubM][2], int mySub,
+                                             int waveRow0, int waveN, int l32, int lhi, int tid,
+                                             const float* ldsRowScale, float* ldsRowMax, Hook afterScaleLoads = NoHook{}) {
+    TileEpilogueWave<kSubM, 2, 0, kTileM, kEpi>(a, t, acc, mySub, waveRow0, waveN, l32, lhi, ldsRowScale, ldsRowMax, afterScaleLoads);
+    if (kEpi == Epilogue::kSwiglu) TileEpilogueFoldMax<kTileM>(a, t, tid, ldsRowMax);
 }
 
 // Calls f(std::integral_constant<int, n>) for n = count clamped into 0..kMax.
@@ -720,11 +741,20 @@ __device__ __forceinline__ void ForCount(int count, F& f) {
 // each has its own issue cursor: at k-step s a wave issues its activation share of step s + 2 and then its weight share
 // of step s + 3.  A wave's loads return in issue order; with the activation share going out first, "at most one weight
 // share outstanding" certifies both the activation stage issued one step ago and the weight stage issued two steps ago.
-template <int kSub0, int kSub1, int kStep>
+//
+// kWn = waves side by side along the channels: four (a wave owns 64 channels, two MFMA column blocks) or two (128
+// channels, four column blocks: with two wave rows that is four waves per workgroup, one per SIMD, each holding a
+// 128 x 128 block of the tile -- a third fewer fragment bytes out of LDS per MFMA, the accumulators in AccVGPRs).
+// Only kWn = 4 is launched.  The four-wave form of the 256-row tile gives the same bits and measured 16 % slower on the
+// matrix-bound shape (4.14 against 3.58 ms): with one wave per SIMD nothing runs under a wave's sixteen operand
+// requests per k-step or under its epilogue, and what it saves in LDS reads is not what bounds the step.
+template <int kSub0, int kSub1, int kStep, int kWn = kWavesN>
 struct StreamCfg {
     static_assert(kSub1 <= kSub0, "wave row 0 is the taller one");
+    static_assert(kWn == 4 || kWn == 2, "a wave owns two or four column blocks");
     static constexpr int kWavesM = kSub1 > 0 ? 2 : 1;
-    static constexpr int kWaves = kWavesN * kWavesM;
+    static constexpr int kWaves = kWn * kWavesM;
+    static constexpr int kNi = kTileN / 32 / kWn;  // MFMA column blocks per wave
     static constexpr int kThreads = 64 * kWaves;
     static constexpr int kTileM = 32 * (kSub0 + kSub1);
     static constexpr int kStageBytesA = kTileM * kStep;
@@ -744,6 +774,7 @@ struct StreamCfg {
     static constexpr int kInstrB = kTileN / kRowsPerInstr;
     static constexpr int kInstr = kInstrA + kInstrB;
     static_assert(kTileM % kRowsPerInstr == 0, "tile rows must fill whole DMA instructions");
+    static_assert(kThreads >= kTileM, "one thread per tile row stages the row scales and folds the row maxima");
     // Every wave issues exactly kMaxPerWave DMA instructions per stage: slots past the last instruction repeat it (same
     // bytes to the same place), which keeps the issue code free of branches and the vmcnt arithmetic uniform.
     static constexpr int kMaxPerWave = (kInstr + kWaves - 1) / kWaves;
@@ -827,13 +858,14 @@ __device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leavi
 // k XOR-ed by 2 * (k & 7), and the operands come out through the same transposing load as for the blocked layout: the
 // 32 lanes the LDS serves together read one pair of neighbouring chunks from each of 8 consecutive k-rows, and the
 // swizzle puts those 8 pairs into 8 different bank groups (a row of 256 bytes spans all 64 banks once).
-template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor = false>
-__global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor = false, int kWn = kWavesN>
+__global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKernel(
     KernelArgs a, const int32_t* __restrict__ sched) {
     static_assert(!(kNz || kNMajor) || kStep == 128, "the blocked and row-major weight layouts are built for 128-byte k-steps");
     static_assert(!(kNz && kNMajor), "one weight layout at a time");
-    using Cfg = StreamCfg<kSub0, kSub1, kStep>;
+    using Cfg = StreamCfg<kSub0, kSub1, kStep, kWn>;
     constexpr int kSubM = kSub0;  // accumulator tiles per wave (wave row 1 uses the first kSub1 of them)
+    constexpr int kNi = Cfg::kNi;
     constexpr int kTileM = Cfg::kTileM;
     constexpr int kStagesA = Cfg::kStagesA, kStagesB = Cfg::kStagesB;
     constexpr int kStageBytesA = Cfg::kStageBytesA, kStageBytesB = Cfg::kStageBytesB;
@@ -851,8 +883,8 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int waveN = wave % kWavesN;
-    const int waveM = wave / kWavesN;
+    const int waveN = wave % kWn;
+    const int waveM = wave / kWn;
     const int l32 = lane & 31;
     const int lhi = lane >> 5;
 
@@ -1142,9 +1174,14 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
     // instantiated once per MFMA-tile count (0..kSub0) so that its body stays straight-line code.
     int waveRow0 = 0;  // first tile row of this wave
     int mySub = 0;     // MFMA tiles of this wave in the current tile
-    const int bRow0 = kSwiglu ? 32 * waveN : 64 * waveN;
-    const int bRowStep = kSwiglu ? kTileN / 2 : 32;
-    v16i acc[kSubM][2];
+    // Row of the weight tile where the wave's column block ni begins.  Blocks come in pairs (2p, 2p + 1) that sit at
+    // column position kNi / 2 * waveN + p of the tile: plain epilogues, the two halves of 64 neighbouring channels;
+    // kSwiglu, 32 activated channels (rows 0..127 of the tile) and their 32 linear partners (rows 128..255).
+    auto bRow = [&](int ni) __attribute__((always_inline)) {
+        const int position = kNi / 2 * waveN + ni / 2;
+        return kSwiglu ? 32 * position + (ni & 1) * (kTileN / 2) : 64 * position + 32 * (ni & 1);
+    };
+    v16i acc[kSubM][kNi];
 
     while (true) {
         const TileInfo following = tileAt(curNo + 1);
@@ -1156,7 +1193,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
 #pragma unroll
         for (int mi = 0; mi < kSubM; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
+            for (int ni = 0; ni < kNi; ++ni)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
 
@@ -1169,7 +1206,7 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
             constexpr int kMy = decltype(myTag)::value;
             constexpr int kSlices = kStep / 32;
             static_assert(kSlices % 2 == 0, "the fragment double buffer is handed over between steps at slot 0");
-            v4i bf[2][2];
+            v4i bf[2][kNi];
             v4i af[2][kMy > 0 ? kMy : 1];
             auto loadSlice = [&](int stageA, int stageB, int ks, int buf) __attribute__((always_inline)) {
                 if (kMy == 0) return;
@@ -1183,8 +1220,8 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                     const int k = 32 * ks + 16 * lhi + (j >> 1);
                     const uint32_t bBase = ldsBase + kFirstB + stageB * kStrideB + 8 * (j & 1);
 #pragma unroll
-                    for (int ni = 0; ni < 2; ++ni) {
-                        const int c = (bRow0 + ni * bRowStep + 16 * ((lane >> 4) & 1)) >> 4;  // logical 16-byte chunk of the row
+                    for (int ni = 0; ni < kNi; ++ni) {
+                        const int c = (bRow(ni) + 16 * ((lane >> 4) & 1)) >> 4;  // logical 16-byte chunk of the row
                         // k and k + 8 share their low three bits, hence their swizzle
                         const uint32_t lo = bBase + k * 256 + ((c ^ ((k & 7) << 1)) << 4);
                         const uint32_t hi = lo + 8 * 256;
@@ -1198,17 +1235,18 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                     const int j = lane & 15;
                     const int inBlock = (32 * ks + 16 * lhi + (j >> 1)) * 32 + 16 * ((lane >> 4) & 1) + 8 * (j & 1);
 #pragma unroll
-                    for (int ni = 0; ni < 2; ++ni) {
+                    for (int ni = 0; ni < kNi; ++ni) {
                         // addressed through the 32-bit LDS address: no generic-to-LDS pointer conversion in the loop
-                        const uint32_t blk = ldsBase + kFirstB + stageB * kStrideB +
-                                             ((bRow0 + ni * bRowStep) >> 5) * 4096 + inBlock;
+                        const uint32_t blk = ldsBase + kFirstB + stageB * kStrideB + (bRow(ni) >> 5) * 4096 + inBlock;
                         const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk));
                         const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LdsV2iPtr>(blk + 8 * 32));
                         bf[buf][ni] = v4i{lo[0], lo[1], hi[0], hi[1]};
                     }
                 } else {
-                    bf[buf][0] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + l32, chunk));
-                    bf[buf][1] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow0 + bRowStep + l32, chunk));
+#pragma unroll
+                    for (int ni = 0; ni < kNi; ++ni) {
+                        bf[buf][ni] = *reinterpret_cast<const v4i*>(B + LdsOffset<kStep>(bRow(ni) + l32, chunk));
+                    }
                 }
 #pragma unroll
                 for (int mi = 0; mi < kMy; ++mi) {
@@ -1243,8 +1281,10 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                     }
 #pragma unroll
                     for (int mi = 0; mi < kMy; ++mi) {
-                        acc[mi][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][0], acc[mi][0], 0, 0, 0);
-                        acc[mi][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][1], acc[mi][1], 0, 0, 0);
+#pragma unroll
+                        for (int ni = 0; ni < kNi; ++ni) {
+                            acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][mi], bf[ks & 1][ni], acc[mi][ni], 0, 0, 0);
+                        }
                     }
                     if constexpr (kEarly && kMy > 0) {
                         if (ks + 1 < kSlices) {
@@ -1253,10 +1293,10 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                             // and, at the register limit of the tallest tiles, on others a late-read order that stalls
                             // the matrix pipe.  (Reading each fragment only when the one before it has retired saves
                             // registers and measures slower.)
-                            constexpr int kReads = kMy + ((kNz || kNMajor) ? 4 : 2);
-                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
-                            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);       // the LDS reads
-                            __builtin_amdgcn_sched_group_barrier(0x008, 2 * kMy - 1, 0);  // the other MFMAs
+                            constexpr int kReads = kMy + ((kNz || kNMajor) ? 2 * kNi : kNi);
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);         // the LDS reads
+                            __builtin_amdgcn_sched_group_barrier(0x008, kNi * kMy - 1, 0);  // the other MFMAs
                         }
                     }
                     if (!kEarly && ks == 0) issueStage();  // into the buffer that the step before read
@@ -1285,7 +1325,13 @@ __global__ __launch_bounds__(kSub1 > 0 ? 512 : 256) void StreamGemmKernel(
                 if (c >= 0) drawValue = QueueTake(a.queueCounters, c);
             }
         };
-        TileEpilogue<kSubM, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, waveN, Opaque(l32), Opaque(lhi), Opaque(tid), ldsRowScale, ldsRowMax, draw);
+        TileEpilogueWave<kSubM, kNi, 0, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, kNi / 2 * waveN, Opaque(l32), Opaque(lhi),
+                                                      ldsRowScale, ldsRowMax, draw);
+        if constexpr (kNi == 4) {
+            TileEpilogueWave<kSubM, kNi, 1, kTileM, kEpi>(a, cur, acc, mySub, waveRow0, kNi / 2 * waveN + 1, Opaque(l32), Opaque(lhi),
+                                                          ldsRowScale, ldsRowMax);
+        }
+        if constexpr (kSwiglu) TileEpilogueFoldMax<kTileM>(a, cur, Opaque(tid), ldsRowMax);
         // Loads and stores may retire out of order with respect to each other, so drain everything (the epilogue's
         // stores and the DMAs in flight, which had the whole epilogue to land) before counting DMAs again.
         WaitVmcnt<0>();
@@ -1519,10 +1565,10 @@ uint64_t* SpanBufferFor(Epilogue epi, int grid, int tileM) {
     return gSpanBuf[k];
 }
 
-template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor>
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor, int kWn = kWavesN>
 hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
-    using Cfg = StreamCfg<kSub0, kSub1, kStep>;
-    auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi, kNz, kNMajor>;
+    using Cfg = StreamCfg<kSub0, kSub1, kStep, kWn>;
+    auto kernel = StreamGemmKernel<kSub0, kSub1, kStep, kEpi, kNz, kNMajor, kWn>;
     static std::atomic<uint64_t> optedIn{0};
     const hipError_t attr = opapi::EnsureDynamicLds(reinterpret_cast<const void*>(kernel), Cfg::kLdsBytes, optedIn);
     if (attr != hipSuccess) return attr;
