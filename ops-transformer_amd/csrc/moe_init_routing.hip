@@ -184,9 +184,9 @@ struct InverseMap {
     int32_t capacity;
     int32_t* gatherIdx;       // gather-type map [destination] -> source, or nullptr
     int32_t dropFrom;         // destinations at or beyond binBase[dropFrom] are dropped (-1 in both maps); < 0: none
-    // One-workgroup sort only: rows of exactly four bytes (a column of per-token scales, say) are copied by the sort
-    // itself -- narrowOut[destination] = narrowX[source / topK] for destinations below activeRows -- which saves the
-    // gather launch of a decode-sized call.  nullptr: rows are gathered by a kernel of their own.
+    // Rows of exactly four bytes (a column of per-token scales, say) are copied by the sort's last scatter itself --
+    // narrowOut[destination] = narrowX[source / topK] for destinations below activeRows -- which saves the gather
+    // launch.  nullptr: rows are gathered by a kernel of their own.
     const uint32_t* narrowX;
     uint32_t* narrowOut;
     int32_t topK;
@@ -229,6 +229,8 @@ __global__ __launch_bounds__(kSortThreads) void DigitScatterKernel(SortPass p, I
                 im.expandedRowIdx[payload] = dropped ? -1 : row;
             }
             if (im.gatherIdx != nullptr) im.gatherIdx[dst] = dropped ? -1 : payload;
+            // four-byte rows ride along with the last pass (see InverseMap)
+            if (im.narrowX != nullptr && !dropped && dst < im.activeRows) im.narrowOut[dst] = im.narrowX[payload / im.topK];
         }
     }
 }
@@ -716,9 +718,9 @@ class InitRoutingExecutor : public aclOpExecutor {
     // key/value pairs and a proper sub-range (whose sentinel bin must not be counted) go through CountV3Kernel.
     bool WideCountsFromScan() const { return v3 && !remap && countMode != 2 && passes == 1; }
 
-    // Decode-sized call on four-byte rows with nothing else riding along: the one-workgroup sort copies the rows itself.
+    // Four-byte rows with nothing else riding along: the sort's last scatter copies the rows itself.
     bool SortCopiesRows() const {
-        return smallSort && rowBytes == 4 && tokens > 0 && !dropPad && scale == nullptr && !dynamicQuant && staticScale == nullptr &&
+        return rowBytes == 4 && tokens > 0 && !dropPad && scale == nullptr && !dynamicQuant && staticScale == nullptr &&
                (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(expandedX)) % 4 == 0;
     }
 
@@ -788,7 +790,7 @@ class InitRoutingExecutor : public aclOpExecutor {
             InverseMap im{last ? expandedRowIdx : nullptr, dropPad, static_cast<int32_t>(capacity),
                           last ? gatherIdxOut : nullptr, (remap && passes == 1) ? expertEnd - expertStart : -1,
                           nullptr, nullptr, static_cast<int32_t>(topK), activeRows};
-            if (SortCopiesRows()) {
+            if (last && SortCopiesRows()) {
                 im.narrowX = reinterpret_cast<const uint32_t*>(x);
                 im.narrowOut = reinterpret_cast<uint32_t*>(expandedX);
             }

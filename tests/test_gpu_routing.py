@@ -382,3 +382,19 @@ def test_quant_v2_outputs_are_rewritten_and_empty_input(aclnn, oracle, dev):
                                             expert_num=E, expert_tokens_count_or_cumsum_flag=1)
     torch.cuda.synchronize()
     assert empty[0].shape == (0, H) and empty[2].cpu().tolist() == [0] * E
+
+
+@pytest.mark.parametrize("T,K,E,active", [(64, 8, 128, 0), (64, 8, 128, 100), (4096, 8, 256, 0), (4096, 8, 256, 5000),
+                                          (3000, 4, 5000, 0), (3000, 4, 5000, 777)])
+@pytest.mark.parametrize("dtype,H", [(np.float32, 1), (np.int8, 4), (np.float16, 2)])
+def test_four_byte_rows_are_copied_by_the_sort(aclnn, oracle, dev, T, K, E, active, dtype, H):
+    """Rows of exactly four bytes (the column of per-token scales that the chain routes with a second call) are written by
+    the sort's last scatter, without a gather launch: one-workgroup sort, three-kernel sort and the two-pass sort of a wide
+    expert range, with and without activeNum cutting the rows off."""
+    rng = np.random.default_rng(T + K + E + active + H)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    x = rng.integers(-100, 100, (T, H)).astype(dtype)
+    ex, ri, cnt, _ = _run(aclnn, dev, x, idx, active_num=active, expert_num=E, expert_tokens_count_or_cumsum_flag=1)
+    ex_r, ri_r, cnt_r, _ = oracle.moe_init_routing_v2(x, idx, active_num=active, expert_num=E, count_flag=1)
+    assert np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r)
+    assert ex.shape == ex_r.shape and np.array_equal(ex.view(np.uint8), ex_r.view(np.uint8))
