@@ -6,17 +6,20 @@
 
 A step is one pass of the path (routing -> gate/up GEMM + SwiGLU + requant -> down GEMM -> finalize) over one batch of
 synthetic tokens whose inputs and expert weights are already resident in HBM.  Prints ONE JSON line: tokens/s for the
-whole pass (K passes between two device synchronisations, nothing else in the stream), the roofline of the dominant
-kernel (the gate/up grouped GEMM) from HIP-event durations recorded inside the library, on the launch stream, during K
-further passes run right after (an event pair around every launch costs the stream ~10 us, which is why the two sets
-of passes are separate; `ms_per_step_kernel_timer_on` reports the second set), and the CPU oracle timed on a bounded
-sample of the same workload.
+whole pass -- the K passes run as --repeats consecutive blocks, each between two device synchronisations with nothing
+else in the stream, and ms_per_step is the median block (fastest, slowest and the mean over all passes are printed
+beside it) --, the rooflines of the two grouped GEMM kernels (`roofline`: the dominant one, gate/up; `roofline_down_gemm`)
+from HIP-event durations recorded inside the library, on the launch stream, during up to 20 further passes run right
+after (an event pair around every launch costs the stream ~10 us, which is why the two sets of passes are separate;
+`ms_per_step_kernel_timer_on` reports the second set), the workspace bytes each operator's first phase asked for, and
+the CPU oracle timed on a bounded sample of the same workload.
 
 The headline (`value`, `roofline`) is the configuration named by --config (default c1, the DeepSeek-V3 prefill shape
-the target is quoted on), run eagerly.  The same line carries, under `other_configs`, a shorter measurement of the other
-halves of the metric: the decode shape c3 (eager and as a HIP-graph replay: HBM-bound), the Mixtral prefill shape c2
-(the MFMA-bound one), the skewed shape c4, and c1 again with aclnnMoeInitRoutingV2 in place of V3 at the head of the
-chain -- each with its ms per pass, per-kernel durations and the gate/up kernel's roofline from the same in-library timer.
+the target is quoted on) behind the routing operator named by --routing (default v2: aclnnMoeInitRoutingV2 on the int8
+rows and on the column of per-token scales), run eagerly.  The same line carries, under `other_configs`, a shorter
+measurement of the other halves of the metric: the decode shape c3 (eager and as a HIP-graph replay: HBM-bound), the
+Mixtral prefill shape c2 (the MFMA-bound one), the skewed shape c4, and c1 again as a graph replay and behind the other
+routing operator -- each with its ms per pass, per-kernel durations and both kernels' rooflines from the same timer.
 
 --calibration-copy appends, after the timed region, a few launches of the library's plain 1 GiB copy kernel: under
 `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` its counter readings give the factor that converts the counters to
