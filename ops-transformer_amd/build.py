@@ -98,7 +98,7 @@ def check_lds_dma_assembly(asm_path):
 def check_ring_kernel_codegen(asm_path):
     """Second build-time guard on the device assembly of grouped_gemm_i8.hip, for three properties of the generated code
     that the kernels' speed and exactness rest on and that a compiler can change without any test noticing at once:
-      * no LDS-ring kernel (StreamGemmKernel) uses scratch memory -- a spilled register is reloaded inside the tile loop;
+      * no LDS-ring kernel (StreamGemmKernel, MixedGemmKernel) uses scratch memory -- a spilled register is reloaded inside the tile loop;
       * no generic (flat) memory instruction: one still in flight makes the compiler drain vmcnt, DMAs included, in
         front of every LDS read;
       * no mixed-precision multiply-add (v_fma_mix*, v_mad_mix*): that is a product and its fp16 conversion merged into
@@ -114,7 +114,7 @@ def check_ring_kernel_codegen(asm_path):
     checked = 0
     for block in text.split(".amdhsa_kernel ")[1:]:
         name = block.split()[0]
-        if "StreamGemmKernel" not in name:
+        if "StreamGemmKernel" not in name and "MixedGemmKernel" not in name:
             continue
         fields = dict(l.split()[:2] for l in block.split(".end_amdhsa_kernel")[0].splitlines()[1:] if len(l.split()) >= 2)
         if int(fields.get(".amdhsa_private_segment_fixed_size", "0")) != 0:

@@ -339,9 +339,11 @@ __device__ __forceinline__ void QueueShare(int64_t tilesBig, int64_t tilesSmall,
 __device__ __forceinline__ int QueueCandidate(int i, int home, int prefer) {
     return 2 * ((home + (i >> 1)) & (kXcds - 1)) + ((i & 1) ? 1 - prefer : prefer);
 }
-__device__ __forceinline__ int QueueFirstOpen(uint32_t usedUp, int home, int prefer) {
+// onlyPreferred: the other run's counters are not candidates at all (a workgroup that serves one run at a time).
+__device__ __forceinline__ int QueueFirstOpen(uint32_t usedUp, int home, int prefer, bool onlyPreferred = false) {
 #pragma unroll
     for (int i = 0; i < 2 * kXcds; ++i) {
+        if (onlyPreferred && (i & 1)) continue;
         const int c = QueueCandidate(i, home, prefer);
         if (((usedUp >> c) & 1u) == 0) return c;
     }
@@ -358,7 +360,7 @@ struct QueueDraw {
     uint32_t usedUp;  // the caller's mask of used-up counters, updated
 };
 __device__ __forceinline__ QueueDraw QueueResolve(int64_t tilesBig, int64_t tilesSmall, int32_t* counters, int home, int prefer,
-                                                  uint32_t usedUp, int c, int32_t v) {
+                                                  uint32_t usedUp, int c, int32_t v, bool onlyPreferred = false) {
     while (c >= 0) {
         int64_t first, size;
         QueueShare(tilesBig, tilesSmall, c, &first, &size);
@@ -373,7 +375,7 @@ __device__ __forceinline__ QueueDraw QueueResolve(int64_t tilesBig, int64_t tile
             QueueShare(tilesBig, tilesSmall, i, &first, &size);
             if (now[i] >= size) usedUp |= 1u << i;
         }
-        c = QueueFirstOpen(usedUp, home, prefer);
+        c = QueueFirstOpen(usedUp, home, prefer, onlyPreferred);
         if (c >= 0) v = QueueTake(counters, c);
     }
     return QueueDraw{-1, 0, usedUp};
@@ -858,9 +860,14 @@ __device__ __forceinline__ void WaitVmcnt() {  // s_waitcnt vmcnt(kCount), leavi
 // k XOR-ed by 2 * (k & 7), and the operands come out through the same transposing load as for the blocked layout: the
 // 32 lanes the LDS serves together read one pair of neighbouring chunks from each of 8 consecutive k-rows, and the
 // swizzle puts those 8 pairs into 8 different bank groups (a row of 256 bytes spans all 64 banks once).
-template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor = false, int kWn = kWavesN>
-__global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKernel(
-    KernelArgs a, const int32_t* __restrict__ sched) {
+//
+// kRun: which runs of the m-tile table the body serves.  kBothRuns: all of it (pulled or in fixed shares).  kBigRun /
+// kSmallRun: that run only, pulled, until its counters are used up on every XCD -- the form in which MixedGemmKernel
+// calls the body twice, once per run with a stage geometry of that run's own.
+constexpr int kBigRun = 0, kSmallRun = 1, kBothRuns = 2;
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor, int kWn, int kRun>
+__device__ __forceinline__ void StreamGemmBody(const KernelArgs& a, const int32_t* __restrict__ sched, char* const lds,
+                                               uint64_t& spanTiles) {
     static_assert(!(kNz || kNMajor) || kStep == 128, "the blocked and row-major weight layouts are built for 128-byte k-steps");
     static_assert(!(kNz && kNMajor), "one weight layout at a time");
     using Cfg = StreamCfg<kSub0, kSub1, kStep, kWn>;
@@ -876,7 +883,6 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
     constexpr int kStrideB = kStaggered ? kStageBytesB : kStageBytesA + kStageBytesB;
     constexpr int kFirstB = kStaggered ? kStagesA * kStageBytesA : kStageBytesA;       // weight part of stage 0
     constexpr bool kSwiglu = kEpi == Epilogue::kSwiglu;
-    extern __shared__ __attribute__((aligned(16))) char lds[];
     float* const ldsRowScale = reinterpret_cast<float*>(lds + kStagesA * kStageBytesA + kStagesB * kStageBytesB);  // [kTileM]
     float* const ldsRowMax = ldsRowScale + kTileM;                                      // [kWavesN][kTileM]
 
@@ -902,7 +908,8 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
     const int xcd = blockIdx.x % kXcds;
     const int32_t slots = gridDim.x / kXcds;
     const int32_t slot = blockIdx.x / kXcds;
-    const bool pull = a.pullTiles != 0;
+    constexpr bool kOneRun = kRun != kBothRuns;
+    const bool pull = kOneRun || a.pullTiles != 0;
     const int64_t bigTiles = static_cast<int64_t>(countBig) * a.tilesN;
     const int64_t totalTiles = bigTiles + static_cast<int64_t>(countSmall) * a.tilesN;
     const int64_t perXcd = (totalTiles + kXcds - 1) / kXcds;
@@ -918,7 +925,7 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
         int64_t forSmall = costAll > 0 ? (slots * costSmall + costAll / 2) / costAll : 0;
         if (forSmall == 0 && countSmall > 0 && slots > 1) forSmall = 1;
         if (countBig == 0) forSmall = slots;
-        prefer = slot < forSmall ? 1 : 0;
+        prefer = kOneRun ? kRun : (slot < forSmall ? 1 : 0);
     }
     auto listTile = [&](int32_t list, int64_t logical) __attribute__((always_inline)) {
         return DecodeListTile<kTileM, kSwiglu>(a, mTileTable, list ? countBig : 0, list ? countSmall : countBig,
@@ -941,13 +948,13 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
         if (tid == 0) {
             // the first two tiles: both draws go out together
             uint32_t usedUp = 0;
-            const int c = QueueFirstOpen(usedUp, xcd, prefer);
+            const int c = QueueFirstOpen(usedUp, xcd, prefer, kOneRun);
             const int32_t v0 = QueueTake(a.queueCounters, c);
             const int32_t v1 = QueueTake(a.queueCounters, c);
-            QueueDraw d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer, usedUp, c, v0);
+            QueueDraw d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer, usedUp, c, v0, kOneRun);
             ldsSeq[0] = d.list;
             ldsSeq[1] = d.logical;
-            if (d.list >= 0) d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer, d.usedUp, c, v1);
+            if (d.list >= 0) d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer, d.usedUp, c, v1, kOneRun);
             ldsSeq[2] = d.list;
             ldsSeq[3] = d.logical;
             ldsSeq[kSeqUsedUp] = static_cast<int32_t>(d.usedUp);
@@ -955,18 +962,9 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
         __syncthreads();
     }
 
-    const uint64_t spanStart = a.wgSpans != nullptr ? __builtin_amdgcn_s_memrealtime() : 0;
-    uint64_t spanTiles = 0;
     int32_t curNo = 0;  // position of the tile being computed in this workgroup's sequence
     TileInfo cur = tileAt(0);
-    if (!cur.valid) {
-        if (a.wgSpans != nullptr && tid == 0) {
-            a.wgSpans[3 * blockIdx.x] = spanStart;
-            a.wgSpans[3 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime();
-            a.wgSpans[3 * blockIdx.x + 2] = 0;
-        }
-        return;
-    }
+    if (!cur.valid) return;
     const int kSteps = a.K / kStep;
     // Small tiles are the decode shapes: a handful of rows per expert, every weight byte used once, pure streaming.
     constexpr bool kSmallTile = kTileM <= 64;
@@ -1320,7 +1318,7 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
         int32_t drawValue = 0;
         auto draw = [&]() __attribute__((always_inline)) {
             if (pull && following.valid && tid == 0) {
-                const int c = QueueFirstOpen(static_cast<uint32_t>(ldsSeq[kSeqUsedUp]), xcd, prefer);
+                const int c = QueueFirstOpen(static_cast<uint32_t>(ldsSeq[kSeqUsedUp]), xcd, prefer, kOneRun);
                 ldsSeq[kSeqDrawCounter] = c;
                 if (c >= 0) drawValue = QueueTake(a.queueCounters, c);
             }
@@ -1339,7 +1337,7 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
         if (!following.valid) break;
         if (pull && tid == 0) {
             const QueueDraw d = QueueResolve(bigTiles, totalTiles - bigTiles, a.queueCounters, xcd, prefer,
-                                             static_cast<uint32_t>(ldsSeq[kSeqUsedUp]), ldsSeq[kSeqDrawCounter], drawValue);
+                                             static_cast<uint32_t>(ldsSeq[kSeqUsedUp]), ldsSeq[kSeqDrawCounter], drawValue, kOneRun);
             ldsSeq[2 * ((curNo + 2) & 3)] = d.list;
             ldsSeq[2 * ((curNo + 2) & 3) + 1] = d.logical;
             ldsSeq[kSeqUsedUp] = static_cast<int32_t>(d.usedUp);
@@ -1349,11 +1347,55 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
         cur = following;
         ++curNo;
     }
-    if (a.wgSpans != nullptr && tid == 0) {
-        a.wgSpans[3 * blockIdx.x] = spanStart;
+}
+
+// Workgroup span record (include/opapi_profile.h): start, end, tiles computed.
+__device__ __forceinline__ void WriteSpan(const KernelArgs& a, uint64_t start, uint64_t tiles) {
+    if (a.wgSpans != nullptr && threadIdx.x == 0) {
+        a.wgSpans[3 * blockIdx.x] = start;
         a.wgSpans[3 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime();
-        a.wgSpans[3 * blockIdx.x + 2] = spanTiles;
+        a.wgSpans[3 * blockIdx.x + 2] = tiles;
     }
+}
+
+template <int kSub0, int kSub1, int kStep, Epilogue kEpi, bool kNz, bool kNMajor = false, int kWn = kWavesN>
+__global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKernel(
+    KernelArgs a, const int32_t* __restrict__ sched) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const uint64_t spanStart = a.wgSpans != nullptr ? __builtin_amdgcn_s_memrealtime() : 0;
+    uint64_t spanTiles = 0;
+    StreamGemmBody<kSub0, kSub1, kStep, kEpi, kNz, kNMajor, kWn, kBothRuns>(a, sched, lds, spanTiles);
+    WriteSpan(a, spanStart, spanTiles);
+}
+
+// 256-row tiles with pulled tiles: the two runs of the m-tile table, each with a stage geometry of its own.  A big
+// m-tile needs 256 activation rows per stage and leaves LDS room for two stages; a small one (at most 64 rows: the
+// whole K x 256 weight block for a handful of rows) needs 64 and runs as a pure weight stream, for which two stages in
+// flight per CU are too few -- with the geometry of the 64-row tiles it has three, the rotated k walk and the
+// non-temporal weight loads of the decode shapes.  A workgroup serves the run it prefers (the small run gets the share
+// of each XCD's workgroups that its cost is of the whole) until that run's counters are used up on every XCD, lets its
+// ring drain, and serves the other; a launch without small m-tiles costs the workgroups that looked for them one draw.
+template <Epilogue kEpi, bool kNz, bool kNMajor>
+__global__ __launch_bounds__(512) void MixedGemmKernel(KernelArgs a, const int32_t* __restrict__ sched) {
+    static_assert(StreamCfg<1, 1, 128>::kTileM == kSmallRows, "the small run's geometry is that of the 64-row tiles");
+    static_assert(StreamCfg<1, 1, 128>::kThreads == 512 && StreamCfg<4, 4, 128>::kThreads == 512, "one workgroup size for both");
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const uint64_t spanStart = a.wgSpans != nullptr ? __builtin_amdgcn_s_memrealtime() : 0;
+    uint64_t spanTiles = 0;
+    const int64_t costSmall = sched[2], costAll = costSmall + sched[3];
+    const int32_t slots = gridDim.x / kXcds, slot = blockIdx.x / kXcds;
+    int64_t forSmall = costAll > 0 ? (slots * costSmall + costAll / 2) / costAll : 0;
+    if (forSmall == 0 && sched[1] > 0 && slots > 1) forSmall = 1;
+    if (slot < forSmall) {
+        StreamGemmBody<1, 1, 128, kEpi, kNz, kNMajor, kWavesN, kSmallRun>(a, sched, lds, spanTiles);
+        __syncthreads();  // the other geometry lays LDS out anew
+        StreamGemmBody<4, 4, 128, kEpi, kNz, kNMajor, kWavesN, kBigRun>(a, sched, lds, spanTiles);
+    } else {
+        StreamGemmBody<4, 4, 128, kEpi, kNz, kNMajor, kWavesN, kBigRun>(a, sched, lds, spanTiles);
+        __syncthreads();
+        StreamGemmBody<1, 1, 128, kEpi, kNz, kNMajor, kWavesN, kSmallRun>(a, sched, lds, spanTiles);
+    }
+    WriteSpan(a, spanStart, spanTiles);
 }
 
 // ---------------------------------------------------------------------------------------------- generic path
@@ -1583,6 +1625,25 @@ hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t ma
     return hipGetLastError();
 }
 
+template <Epilogue kEpi, bool kNz, bool kNMajor>
+hipError_t LaunchMixed(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
+    using Big = StreamCfg<4, 4, 128>;
+    using Small = StreamCfg<1, 1, 128>;
+    constexpr int kLdsBytes = Big::kLdsBytes > Small::kLdsBytes ? Big::kLdsBytes : Small::kLdsBytes;
+    auto kernel = MixedGemmKernel<kEpi, kNz, kNMajor>;
+    static std::atomic<uint64_t> optedIn{0};
+    const hipError_t attr = opapi::EnsureDynamicLds(reinterpret_cast<const void*>(kernel), kLdsBytes, optedIn);
+    if (attr != hipSuccess) return attr;
+    int64_t grid = DeviceCuCount();
+    if (grid > maxTiles) grid = maxTiles;
+    grid = grid / kXcds * kXcds;
+    if (grid < kXcds) grid = kXcds;
+    KernelArgs launchArgs = args;
+    launchArgs.wgSpans = SpanBufferFor(kEpi, static_cast<int>(grid), Big::kTileM);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(512), kLdsBytes, stream, launchArgs, sched);
+    return hipGetLastError();
+}
+
 // Tile heights and their (wave row 0, wave row 1, k-step) shapes.  Up to 192 rows the weight ring holds three or more
 // 128-byte stages; from 192 rows on the activation ring holds two.
 template <Epilogue kEpi, bool kNz, bool kNMajor>
@@ -1594,7 +1655,10 @@ hipError_t LaunchStreamShapeOf(const Plan& plan, const KernelArgs& args, const i
         case 128: return LaunchStream<2, 2, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
         case 160: return LaunchStream<3, 2, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
         case 192: return LaunchStream<3, 3, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
-        default: return LaunchStream<4, 4, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        default:
+            // pulled 256-row tiles: the two runs of the table with a stage geometry each
+            if (plan.pullTiles) return LaunchMixed<kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+            return LaunchStream<4, 4, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
     }
 }
 
