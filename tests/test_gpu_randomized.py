@@ -211,3 +211,54 @@ def test_routing_quant_v2_random(aclnn, oracle, dev, seed):
         assert (g is None) == (w is None), label
         if g is not None:
             assert np.array_equal(_np(g), w), (label, quant, kw, T, K, E, H, name)
+
+
+@pytest.mark.parametrize("seed", SEEDS[:16])
+def test_pulled_skewed_gemm_random(aclnn, oracle, dev, seed):
+    """Tiles of eight k-steps and more with a skewed group list: the workgroups pull their tiles from the counters, and
+    where the planner picks 256-row tiles the two runs of the m-tile table (big, small) run with a stage geometry each.
+    Zipf-like group sizes (a few groups with most of the rows, many with a handful, some empty), all three epilogues,
+    the three weight layouts, cumsum and count lists."""
+    rng = np.random.default_rng(9000 + seed)
+    K = int(rng.choice([1024, 1152, 2048]))
+    N = int(rng.choice([256, 512, 1280]))
+    E = int(rng.choice([3, 8, 24, 40]))
+    M = int(rng.integers(300, 3000))
+    weights = 1.0 / np.arange(1, E + 1) ** float(rng.choice([1.0, 1.5, 2.5]))
+    rng.shuffle(weights)
+    sizes = rng.multinomial(M, weights / weights.sum())
+    sizes[rng.integers(0, E)] = 0
+    cumsum = np.cumsum(sizes).astype(np.int64)
+    M = int(cumsum[-1])
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)          # K-contiguous storage [E, N, K]
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    per_token = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    layout = ["kmajor", "nd", "nz"][seed % 3]
+    w_dev = t(wt)
+    if layout == "kmajor":
+        wkw, wv, w_swiglu = {}, [w_dev.transpose(1, 2)], dict(weight=w_dev.transpose(1, 2))
+    elif layout == "nd":
+        w_nd = w_dev.transpose(1, 2).contiguous()
+        wkw, wv, w_swiglu = {}, [w_nd], dict(weight=w_nd)
+    else:
+        w_nz = w_dev.view(E, N // 32, 32, K // 16, 16).permute(0, 1, 3, 4, 2).contiguous()
+        wkw, wv, w_swiglu = dict(weight_nz=(w_nz, "nz5d")), None, dict(weight=None, weight_nz=(w_nz, "nz5d"))
+    list_type = seed % 2
+    gld = t(cumsum if list_type == 0 else sizes.astype(np.int64))
+    kw = dict(split_item=3, group_type=0, group_list_type=list_type, **wkw)
+
+    acc = aclnn.grouped_matmul_v4([t(x)], wv, group_list=gld, **kw)[0]
+    y = aclnn.grouped_matmul_v4([t(x)], wv, scale=[t(scale)], per_token_scale=[t(per_token)], group_list=gld,
+                                output_dtype=torch.bfloat16, **kw)[0]
+    h, hs = aclnn.grouped_matmul_swiglu_quant(t(x), w_swiglu["weight"], t(cumsum), t(scale), t(per_token),
+                                              **{k: v for k, v in w_swiglu.items() if k != "weight"})
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), oracle.grouped_matmul_i32(x, wt, cumsum, w_trans=True)), (M, K, N, E, layout)
+    ref = oracle.grouped_matmul_dequant(x, wt, scale, per_token, cumsum, w_trans=True, out_dtype=oracle.DT_BF16)
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+    h_r, hs_r = oracle.grouped_matmul_swiglu_quant(x, wt, scale, per_token, cumsum, w_trans=True)
+    diff = np.abs(h.cpu().numpy().astype(np.int32) - h_r.astype(np.int32))
+    assert diff.max(initial=0) <= 1 and (diff != 0).mean() < 1e-2
+    np.testing.assert_allclose(hs.cpu().numpy(), hs_r, rtol=1e-5)
