@@ -1368,17 +1368,17 @@ __global__ __launch_bounds__(64 * kWn * (kSub1 > 0 ? 2 : 1)) void StreamGemmKern
     WriteSpan(a, spanStart, spanTiles);
 }
 
-// 256-row tiles with pulled tiles: the two runs of the m-tile table, each with a stage geometry of its own.  A big
-// m-tile needs 256 activation rows per stage and leaves LDS room for two stages; a small one (at most 64 rows: the
-// whole K x 256 weight block for a handful of rows) needs 64 and runs as a pure weight stream, for which two stages in
-// flight per CU are too few -- with the geometry of the 64-row tiles it has three, the rotated k walk and the
-// non-temporal weight loads of the decode shapes.  A workgroup serves the run it prefers (the small run gets the share
+// Tall tiles (192 and 256 rows) with pulled tiles: the two runs of the m-tile table, each with a stage geometry of its
+// own.  A big m-tile of 256 rows needs 256 activation rows per stage and leaves LDS room for two stages; a small one (at
+// most 64 rows: the whole K x 256 weight block for a handful of rows) needs 64 and runs as a pure weight stream, for
+// which two stages in flight per CU are too few -- with the geometry of the 64-row tiles it has three, the rotated k
+// walk and the non-temporal weight loads of the decode shapes.  A workgroup serves the run it prefers (the small run gets the share
 // of each XCD's workgroups that its cost is of the whole) until that run's counters are used up on every XCD, lets its
 // ring drain, and serves the other; a launch without small m-tiles costs the workgroups that looked for them one draw.
-template <Epilogue kEpi, bool kNz, bool kNMajor>
+template <int kSub0, int kSub1, Epilogue kEpi, bool kNz, bool kNMajor>
 __global__ __launch_bounds__(512) void MixedGemmKernel(KernelArgs a, const int32_t* __restrict__ sched) {
     static_assert(StreamCfg<1, 1, 128>::kTileM == kSmallRows, "the small run's geometry is that of the 64-row tiles");
-    static_assert(StreamCfg<1, 1, 128>::kThreads == 512 && StreamCfg<4, 4, 128>::kThreads == 512, "one workgroup size for both");
+    static_assert(StreamCfg<1, 1, 128>::kThreads == 512 && StreamCfg<kSub0, kSub1, 128>::kThreads == 512, "one workgroup size for both");
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const uint64_t spanStart = a.wgSpans != nullptr ? __builtin_amdgcn_s_memrealtime() : 0;
     uint64_t spanTiles = 0;
@@ -1389,9 +1389,9 @@ __global__ __launch_bounds__(512) void MixedGemmKernel(KernelArgs a, const int32
     if (slot < forSmall) {
         StreamGemmBody<1, 1, 128, kEpi, kNz, kNMajor, kWavesN, kSmallRun>(a, sched, lds, spanTiles);
         __syncthreads();  // the other geometry lays LDS out anew
-        StreamGemmBody<4, 4, 128, kEpi, kNz, kNMajor, kWavesN, kBigRun>(a, sched, lds, spanTiles);
+        StreamGemmBody<kSub0, kSub1, 128, kEpi, kNz, kNMajor, kWavesN, kBigRun>(a, sched, lds, spanTiles);
     } else {
-        StreamGemmBody<4, 4, 128, kEpi, kNz, kNMajor, kWavesN, kBigRun>(a, sched, lds, spanTiles);
+        StreamGemmBody<kSub0, kSub1, 128, kEpi, kNz, kNMajor, kWavesN, kBigRun>(a, sched, lds, spanTiles);
         __syncthreads();
         StreamGemmBody<1, 1, 128, kEpi, kNz, kNMajor, kWavesN, kSmallRun>(a, sched, lds, spanTiles);
     }
@@ -1625,12 +1625,12 @@ hipError_t LaunchStream(const KernelArgs& args, const int32_t* sched, int64_t ma
     return hipGetLastError();
 }
 
-template <Epilogue kEpi, bool kNz, bool kNMajor>
+template <int kSub0, int kSub1, Epilogue kEpi, bool kNz, bool kNMajor>
 hipError_t LaunchMixed(const KernelArgs& args, const int32_t* sched, int64_t maxTiles, hipStream_t stream) {
-    using Big = StreamCfg<4, 4, 128>;
+    using Big = StreamCfg<kSub0, kSub1, 128>;
     using Small = StreamCfg<1, 1, 128>;
     constexpr int kLdsBytes = Big::kLdsBytes > Small::kLdsBytes ? Big::kLdsBytes : Small::kLdsBytes;
-    auto kernel = MixedGemmKernel<kEpi, kNz, kNMajor>;
+    auto kernel = MixedGemmKernel<kSub0, kSub1, kEpi, kNz, kNMajor>;
     static std::atomic<uint64_t> optedIn{0};
     const hipError_t attr = opapi::EnsureDynamicLds(reinterpret_cast<const void*>(kernel), kLdsBytes, optedIn);
     if (attr != hipSuccess) return attr;
@@ -1653,11 +1653,16 @@ hipError_t LaunchStreamShapeOf(const Plan& plan, const KernelArgs& args, const i
         case 64: return LaunchStream<1, 1, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
         case 96: return LaunchStream<2, 1, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
         case 128: return LaunchStream<2, 2, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        // (160-row tiles were measured in the two-geometry form as well: the down projection of the DeepSeek-V3 prefill
+        // shape, whose few overflowing experts leave small second m-tiles, 0.834 against 0.820 ms -- sixteen k-steps
+        // per tile do not repay a change of geometry)
         case 160: return LaunchStream<3, 2, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
-        case 192: return LaunchStream<3, 3, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+        // pulled tiles of 192 and 256 rows: the two runs of the table with a stage geometry each
+        case 192:
+            if (plan.pullTiles) return LaunchMixed<3, 3, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+            return LaunchStream<3, 3, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
         default:
-            // pulled 256-row tiles: the two runs of the table with a stage geometry each
-            if (plan.pullTiles) return LaunchMixed<kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
+            if (plan.pullTiles) return LaunchMixed<4, 4, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
             return LaunchStream<4, 4, 128, kEpi, kNz, kNMajor>(args, sched, plan.maxTiles, stream);
     }
 }
