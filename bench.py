@@ -42,7 +42,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gmm_swiglu_{config}_hbm_traffic.txt")
-KERNEL_SOURCES = ["grouped_gemm_i8.hip", "grouped_gemm_i8.h", "opapi_common.h"]
+KERNEL_SOURCES = ["grouped_gemm_i8.hip", "grouped_gemm_i8_kernels.h", "grouped_gemm_i8.h", "opapi_common.h"]
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA (5.0 POP/s)
 

@@ -24,6 +24,9 @@ SOURCES = [
     "moe_gating_top_k_softmax_v2.hip",
     "moe_init_routing.hip",
     "grouped_gemm_i8.hip",
+    "grouped_gemm_i8_int32.hip",
+    "grouped_gemm_i8_dequant.hip",
+    "grouped_gemm_i8_swiglu.hip",
     "grouped_matmul_swiglu_quant.hip",
     "grouped_matmul_v4.hip",
     "grouped_matmul_finalize_routing.hip",
@@ -43,7 +46,11 @@ COMMON_FLAGS = [
 ]
 
 
-# The LDS-DMA loads of grouped_gemm_i8.hip set m0 in an inline-assembly statement and count outstanding loads by hand,
+# The translation units that hold the LDS-DMA kernels (grouped_gemm_i8_kernels.h instantiated per epilogue): their device
+# assembly goes through the guards below whenever they are compiled.
+RING_SOURCES = ("grouped_gemm_i8_int32.hip", "grouped_gemm_i8_dequant.hip", "grouped_gemm_i8_swiglu.hip")
+
+# The LDS-DMA loads of grouped_gemm_i8_kernels.h set m0 in an inline-assembly statement and count outstanding loads by hand,
 # which leans on how this compiler schedules around such statements.  The kernels were validated (bit-exact suites on
 # the GPU) with the compiler named here; another one has to be validated again before its build is trusted:
 # OPAPI_ALLOW_UNVALIDATED_COMPILER=1 lets the build through so that the suites can be run.
@@ -63,14 +70,14 @@ def check_compiler():
     if any(tag in version for tag in VALIDATED_COMPILERS) or os.environ.get("OPAPI_ALLOW_UNVALIDATED_COMPILER") == "1":
         return version
     raise RuntimeError(
-        "hipcc reports '%s', but the LDS-DMA kernels of grouped_gemm_i8.hip (m0 set in inline assembly, hand-counted "
+        "hipcc reports '%s', but the LDS-DMA kernels of grouped_gemm_i8_kernels.h (m0 set in inline assembly, hand-counted "
         "s_waitcnt vmcnt) were validated with %s only. Set OPAPI_ALLOW_UNVALIDATED_COMPILER=1 to build anyway, run "
         "`pytest tests -m gpu` on an MI355X, and add the compiler to VALIDATED_COMPILERS in %s when the suites are green."
         % (version, " / ".join(VALIDATED_COMPILERS), os.path.abspath(__file__)))
 
 
 def check_lds_dma_assembly(asm_path):
-    """Build-time guard on the device assembly of grouped_gemm_i8.hip: every instruction that writes m0 must be the
+    """Build-time guard on the device assembly of the GEMM kernel units: every instruction that writes m0 must be the
     `s_mov_b32 m0, sN` of an LDS-DMA statement, i.e. be followed at once by its global_load_lds_dwordx4, and every such
     load must be preceded by its own m0 write.  A compiler that puts anything between the two, or writes m0 for a
     purpose of its own inside these kernels, fails the build instead of producing kernels that read stale tiles."""
@@ -96,7 +103,7 @@ def check_lds_dma_assembly(asm_path):
 
 
 def check_ring_kernel_codegen(asm_path):
-    """Second build-time guard on the device assembly of grouped_gemm_i8.hip, for three properties of the generated code
+    """Second build-time guard on the device assembly of the GEMM kernel units, for three properties of the generated code
     that the kernels' speed and exactness rest on and that a compiler can change without any test noticing at once:
       * no LDS-ring kernel (StreamGemmKernel, MixedGemmKernel) uses scratch memory -- a spilled register is reloaded inside the tile loop;
       * no generic (flat) memory instruction: one still in flight makes the compiler drain vmcnt, DMAs included, in
@@ -143,7 +150,7 @@ def _compile(src, force):
     # the object is then marked unguarded and a later build without the variable compiles it again.
     guard_stamp = obj + ".guard-passed"
     unguarded_ok = os.environ.get("OPAPI_ASM_GUARD") == "0"
-    is_ring_source = src == "grouped_gemm_i8.hip"
+    is_ring_source = src in RING_SOURCES
     if is_ring_source and not force and not unguarded_ok and os.path.exists(obj) and not os.path.exists(guard_stamp):
         os.remove(obj)  # built without the guards: not to be linked
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
@@ -152,7 +159,7 @@ def _compile(src, force):
     if is_ring_source and os.path.exists(guard_stamp):
         os.remove(guard_stamp)
     if is_ring_source and not guarded:
-        sys.stderr.write("build.py: OPAPI_ASM_GUARD=0 -- grouped_gemm_i8.hip is compiled WITHOUT the assembly guards\n")
+        sys.stderr.write("build.py: OPAPI_ASM_GUARD=0 -- %s is compiled WITHOUT the assembly guards\n" % src)
     cmd = [HIPCC] + COMMON_FLAGS + (["-save-temps=obj"] if guarded else []) + \
           (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", src_path, "-o", obj]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -179,12 +186,12 @@ def _compile(src, force):
 
 
 # Host-side sanitizer build (AddressSanitizer + UndefinedBehaviorSanitizer on the host pass only; device code is compiled
-# as usual and GPU sanitizers are never involved).  grouped_gemm_i8.hip, whose host part is a few lines of planning
-# around minutes of kernel compilation, is linked from the regular build.
+# as usual and GPU sanitizers are never involved).  The per-epilogue GEMM units, whose host part is a few lines of dispatch
+# around minutes of kernel compilation, are linked from the regular build.
 SANITIZED_LIB_PATH = os.path.join(LIB_DIR, "sanitized", "libcust_opapi.so")
 SANITIZE_FLAGS = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
                   "-Xarch_host", "-fno-sanitize-recover=undefined", "-Xarch_host", "-fno-omit-frame-pointer", "-g"]
-UNSANITIZED = {"grouped_gemm_i8.hip"}
+UNSANITIZED = set(RING_SOURCES)
 
 
 def sanitizer_runtime():
@@ -198,7 +205,7 @@ def sanitizer_runtime():
 
 def build_sanitized(jobs=None):
     """Builds lib/sanitized/libcust_opapi.so: same sources, host code instrumented.  Returns its path."""
-    build()  # the regular objects (grouped_gemm_i8.o is reused)
+    build()  # the regular objects (those of the GEMM kernel units are reused)
     obj_dir = os.path.join(OBJ_DIR, "sanitized")
     os.makedirs(obj_dir, exist_ok=True)
     os.makedirs(os.path.dirname(SANITIZED_LIB_PATH), exist_ok=True)
