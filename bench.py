@@ -96,7 +96,8 @@ def _cpu_baseline(pkg, oracle, cfg, idx, wgt, xq, xs, ffn, sample_experts=4):
 
 
 def _recorded_traffic(config_name):
-    """(bytes per launch or None, description) of the gate/up GEMM's HBM traffic from the committed counter summary.
+    """(bytes or None, description) of the gate/up GEMM's HBM traffic from the committed counter summary: per launch,
+    times the launches of one pass where the operator runs in row bands (like `kernel_ms`).
 
     The summary carries "traffic_bytes_per_launch: N" and "kernel_source_sha256: H" (hash of the kernel sources the
     counters were read on, see kernel_source_hash); a figure taken on other sources is not reported."""
@@ -119,11 +120,14 @@ def _recorded_traffic(config_name):
     return value, src
 
 
-def _kernel_roofline(name, kernel, timer_name, nbytes, ops, kernels, traffic=None, traffic_source=None):
+def _kernel_roofline(name, kernel, timer_name, nbytes, ops, kernels, passes, traffic=None, traffic_source=None):
     """Roofline block of one grouped GEMM kernel from the library's event timer: both fractions, and as `bound` the
-    roof that is the lower one for the kernel's algorithmic bytes and ops."""
+    roof that is the lower one for the kernel's algorithmic bytes and ops.  The bytes and ops are those of the operator's
+    GEMM over all rows; where the operator runs in row bands (the SwiGLU operator above 512 MiB of fp32 result) its
+    kernel is launched once per band, `launches_per_pass` says how often, and `kernel_ms` is the sum over the bands of
+    one pass, i.e. the average launch duration times `launches_per_pass`."""
     n, total = kernels.get(timer_name, (0, 0.0))
-    ms = total / max(n, 1)
+    ms = total / max(passes, 1)
     hbm_frac = nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if ms > 0 else None
     mfma_frac = ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS if ms > 0 else None
     t_hbm = nbytes / (HBM_PEAK_GBS * 1e9)
@@ -136,29 +140,30 @@ def _kernel_roofline(name, kernel, timer_name, nbytes, ops, kernels, traffic=Non
                     "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": traffic}
     if traffic_source is not None:
         roofline["traffic_source"] = traffic_source
-    roofline.update({"kernel": kernel, "kernel_ms": ms, "launches_timed": n, "algorithmic_bytes": nbytes,
+    roofline.update({"kernel": kernel, "kernel_ms": ms, "launches_timed": n, "launches_per_pass": n / float(max(passes, 1)),
+                     "algorithmic_bytes": nbytes,
                      "algorithmic_ops": ops, "hbm_frac": hbm_frac, "mfma_frac": mfma_frac,
                      "time_at_hbm_peak_ms": t_hbm * 1e3, "time_at_mfma_peak_ms": t_mfma * 1e3})
     return roofline
 
 
-def _gate_up_roofline(cfg, touched, kernels):
+def _gate_up_roofline(cfg, touched, kernels, passes):
     """Gate/up grouped GEMM.  Algorithmic bytes of one launch: the touched experts' gate/up weights and channel scales,
     the expanded int8 rows and their scales in, the int8 activations and their scales out.  Ops: 4 * M * H * I."""
     M, H, I = cfg.tokens * cfg.top_k, cfg.hidden, cfg.inter
     nbytes = touched * 2 * H * I + touched * 2 * I * 4 + M * H + M * 4 + M * I + M * 4
     traffic, traffic_source = _recorded_traffic(cfg.name)
     return _kernel_roofline("gate_up", "StreamGemmKernel<..., kSwiglu> (gate/up GEMM + SwiGLU; timer name gmm_swiglu)",
-                            "gmm_swiglu", nbytes, 4 * M * H * I, kernels, traffic, traffic_source)
+                            "gmm_swiglu", nbytes, 4 * M * H * I, kernels, passes, traffic, traffic_source)
 
 
-def _down_roofline(cfg, touched, kernels):
+def _down_roofline(cfg, touched, kernels, passes):
     """Down-projection grouped GEMM.  Algorithmic bytes of one launch: the touched experts' down weights and channel
     scales, the int8 activations and their scales in, the bf16 rows out.  Ops: 2 * M * H * I."""
     M, H, I = cfg.tokens * cfg.top_k, cfg.hidden, cfg.inter
     nbytes = touched * H * I + touched * H * 4 + M * I + M * 4 + M * H * 2
     return _kernel_roofline("down", "StreamGemmKernel<..., kDequant> (down GEMM + dequant; timer name gmm_dequant)",
-                            "gmm_dequant", nbytes, 2 * M * H * I, kernels)
+                            "gmm_dequant", nbytes, 2 * M * H * I, kernels, passes)
 
 
 class Workload:
@@ -256,8 +261,8 @@ class Workload:
                            "hbm_frac": work["bytes"] / sec_per_pass / 1e9 / HBM_PEAK_GBS,
                            "algorithmic_ops": work["ops"], "algorithmic_bytes": work["bytes"]},
             "kernels_ms": {k: v[1] / float(measured["timer_steps"]) for k, v in sorted(kernels.items())},
-            "roofline": _gate_up_roofline(cfg, self.touched, kernels),
-            "roofline_down_gemm": _down_roofline(cfg, self.touched, kernels),
+            "roofline": _gate_up_roofline(cfg, self.touched, kernels, measured["timer_steps"]),
+            "roofline_down_gemm": _down_roofline(cfg, self.touched, kernels, measured["timer_steps"]),
             "workspace_bytes": dict(self.ffn.workspace.requested, allocated=int(self.ffn.workspace.tensor.numel())
                                     if self.ffn.workspace.tensor is not None else 0),
             "gemm_tile_balance": self._tile_balance(),

@@ -62,6 +62,7 @@ struct Plan {
     int32_t maxMTiles = 0;  // upper bound on m-tiles over all groups (M / tileM + groups)
     int32_t tilesN = 0;
     bool pullTiles = false; // LDS-ring kernels: workgroups draw their tiles from counters instead of walking fixed shares
+    int64_t bandRows = 0;   // kSwiglu: rows of S held in the workspace at a time (M when the launch runs as one band)
     uint64_t offSched = 0, offRowMax = 0, offS = 0;
     uint64_t workspaceBytes = 0;
 };

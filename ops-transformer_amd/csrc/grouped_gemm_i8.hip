@@ -48,6 +48,7 @@ struct SchedArgs {
     int32_t tileM;
     int32_t maxMTiles;
     int64_t M;
+    int64_t rowBegin, rowEnd;  // only rows in [rowBegin, rowEnd) get tiles (one band of a launch that runs in row bands)
 };
 
 __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
@@ -138,6 +139,9 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
     }
     begin = begin < 0 ? 0 : (begin > a.M ? a.M : begin);
     end = end < begin ? begin : (end > a.M ? a.M : end);
+    // the band of rows this launch covers: a group keeps the part of its rows that lies inside
+    begin = begin < a.rowBegin ? a.rowBegin : (begin > a.rowEnd ? a.rowEnd : begin);
+    end = end < a.rowBegin ? a.rowBegin : (end > a.rowEnd ? a.rowEnd : end);
     const int32_t rows = t < a.groups ? static_cast<int32_t>(end - begin) : 0;
     const int32_t tiles = (rows + a.tileM - 1) / a.tileM;
     // big and small m-tiles of this group (with tiles of at most kSmallRows rows every m-tile is small; otherwise only
@@ -219,7 +223,7 @@ __global__ __launch_bounds__(1024) void ScheduleKernel(SchedArgs a) {
 
 // ---------------------------------------------------------------------------------------------- requantisation
 struct RequantArgs {
-    const float* s;          // [M, halfN]
+    const float* s;          // [rows of the band, halfN]: row r of the problem at index r - rowBegin
     const float* rowMax;     // [tilesN][M] partial max |S|
     int32_t tilesN;
     int64_t M;
@@ -227,6 +231,7 @@ struct RequantArgs {
     int8_t* y;               // [M, halfN]
     float* yScale;           // [M]
     int32_t halfN;
+    int64_t rowBegin;        // first row of the band; the grid covers the band's rows
 };
 
 __device__ __forceinline__ int8_t QuantOne(float s, float inv) {
@@ -238,10 +243,10 @@ __device__ __forceinline__ int8_t QuantOne(float s, float inv) {
 // Every thread requests its first two packets of S before the row maximum is known, and every wave folds the partial
 // maxima for itself (a handful of L2 hits): the row's two dependent memory round trips overlap and there is no barrier.
 __global__ __launch_bounds__(256) void RequantKernel(RequantArgs a) {
-    const int64_t row = blockIdx.x;
+    const int64_t row = a.rowBegin + blockIdx.x;
     if (row >= a.sched[kHdrCoveredRows]) return;
     typedef float Float4 __attribute__((ext_vector_type(4)));
-    const float* src = a.s + row * a.halfN;
+    const float* src = a.s + static_cast<int64_t>(blockIdx.x) * a.halfN;
     int8_t* dst = a.y + row * a.halfN;
     const bool packets = (a.halfN & 3) == 0;
     constexpr int kAhead = 2;
@@ -399,8 +404,22 @@ Plan MakePlan(const Problem& p) {
     if (p.epilogue == Epilogue::kSwiglu) {
         plan.offRowMax = off;
         off += Align256(static_cast<uint64_t>(p.M) * 4 * static_cast<uint64_t>(plan.tilesN));
+        // S, the fp32 SwiGLU result that the requantisation reads back, is held for one band of rows at a time: at most
+        // 512 MiB of it (OPAPI_SWIGLU_WORKSPACE_MB=<n> sets another limit), in whole m-tiles, at least one.  A launch
+        // whose S fits runs as one band; a taller one runs schedule, GEMM and requantisation once per band.  A band of
+        // 512 MiB is at least 4096 tiles, sixteen rounds of the machine, whatever the shape: measured against a single
+        // band on 1.9 GB of S it costs nothing (halving the limit twice costs 2 % and 7 % of the pass).
+        uint64_t capBytes = 512ull << 20;
+        if (const char* env = std::getenv("OPAPI_SWIGLU_WORKSPACE_MB")) {
+            const long long mb = std::atoll(env);
+            if (mb > 0) capBytes = static_cast<uint64_t>(mb) << 20;
+        }
+        const uint64_t rowBytes = static_cast<uint64_t>(p.N / 2) * 4;
+        int64_t bandRows = rowBytes > 0 ? static_cast<int64_t>(capBytes / rowBytes) / plan.tileM * plan.tileM : p.M;
+        if (bandRows < plan.tileM) bandRows = plan.tileM;
+        plan.bandRows = bandRows < p.M ? bandRows : p.M;
         plan.offS = off;
-        off += Align256(static_cast<uint64_t>(p.M) * static_cast<uint64_t>(p.N / 2) * 4);
+        off += Align256(static_cast<uint64_t>(plan.bandRows) * rowBytes);
     }
     plan.workspaceBytes = off;
     return plan;
@@ -427,10 +446,6 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     sa.tileM = plan.tileM;
     sa.maxMTiles = plan.maxMTiles;
     sa.M = p.M;
-    {
-        opapi::KernelTimer timer("gmm_schedule", stream);
-        hipLaunchKernelGGL(ScheduleKernel, dim3(1), dim3(1024), 0, stream, sa);
-    }
 
     KernelArgs ka{};
     ka.x = p.x;
@@ -463,29 +478,48 @@ hipError_t Enqueue(const Problem& p, const Plan& plan, void* workspace, hipStrea
     ka.pullTiles = plan.pullTiles ? 1 : 0;
 
     hipError_t e = hipSuccess;
-    if (p.K > 0) {
-        const bool fast = StreamOk(p);
-        opapi::KernelTimer timer(p.epilogue == Epilogue::kSwiglu ? "gmm_swiglu"
-                                 : p.epilogue != Epilogue::kDequant ? "gmm_int32"
-                                 : p.combineIndex != nullptr ? "gmm_combine" : "gmm_dequant", stream);
-        switch (p.epilogue) {
-            case Epilogue::kInt32:
-                e = fast ? LaunchRingInt32(plan, ka, sched, stream) : LaunchGenericInt32(plan, ka, sched, stream);
-                break;
-            case Epilogue::kDequant:
-                e = fast ? LaunchRingDequant(plan, ka, sched, stream) : LaunchGenericDequant(plan, ka, sched, stream);
-                break;
-            case Epilogue::kSwiglu:
-                e = fast ? LaunchRingSwiglu(plan, ka, sched, stream) : LaunchGenericSwiglu(plan, ka, sched, stream);
-                break;
+    // One band covers every row unless S is held for a band of rows at a time (kSwiglu with a capped workspace): then
+    // schedule, GEMM and requantisation run once per band, the schedule handing out only the band's rows, and S is
+    // addressed as if the band's first row were at sBuf (the kernels index S by the row of the problem).
+    const int64_t bandRows = swiglu && plan.bandRows > 0 ? plan.bandRows : p.M;
+    for (int64_t rowBegin = 0; rowBegin < p.M; rowBegin += bandRows) {
+        const int64_t rowEnd = rowBegin + bandRows < p.M ? rowBegin + bandRows : p.M;
+        sa.rowBegin = rowBegin;
+        sa.rowEnd = rowEnd;
+        {
+            opapi::KernelTimer timer("gmm_schedule", stream);
+            hipLaunchKernelGGL(ScheduleKernel, dim3(1), dim3(1024), 0, stream, sa);
         }
-        if (e != hipSuccess) return e;
-    }
-    if (swiglu) {
-        RequantArgs ra{sBuf, rowMax, plan.tilesN, p.M, sched, p.quantOut, p.quantScaleOut, static_cast<int32_t>(p.N / 2)};
-        opapi::KernelTimer timer("gmm_requant", stream);
-        hipLaunchKernelGGL(RequantKernel, dim3(static_cast<unsigned>(p.M)), dim3(256), 0, stream, ra);
-        e = hipGetLastError();
+        if (swiglu) {
+            ka.sOut = reinterpret_cast<float*>(reinterpret_cast<uintptr_t>(sBuf) -
+                                               static_cast<uintptr_t>(rowBegin) * static_cast<uintptr_t>(p.N / 2) * 4);
+        }
+        if (p.K > 0) {
+            const bool fast = StreamOk(p);
+            opapi::KernelTimer timer(p.epilogue == Epilogue::kSwiglu ? "gmm_swiglu"
+                                     : p.epilogue != Epilogue::kDequant ? "gmm_int32"
+                                     : p.combineIndex != nullptr ? "gmm_combine" : "gmm_dequant", stream);
+            switch (p.epilogue) {
+                case Epilogue::kInt32:
+                    e = fast ? LaunchRingInt32(plan, ka, sched, stream) : LaunchGenericInt32(plan, ka, sched, stream);
+                    break;
+                case Epilogue::kDequant:
+                    e = fast ? LaunchRingDequant(plan, ka, sched, stream) : LaunchGenericDequant(plan, ka, sched, stream);
+                    break;
+                case Epilogue::kSwiglu:
+                    e = fast ? LaunchRingSwiglu(plan, ka, sched, stream) : LaunchGenericSwiglu(plan, ka, sched, stream);
+                    break;
+            }
+            if (e != hipSuccess) return e;
+        }
+        if (swiglu) {
+            RequantArgs ra{sBuf, rowMax, plan.tilesN, p.M, sched, p.quantOut, p.quantScaleOut, static_cast<int32_t>(p.N / 2),
+                           rowBegin};
+            opapi::KernelTimer timer("gmm_requant", stream);
+            hipLaunchKernelGGL(RequantKernel, dim3(static_cast<unsigned>(rowEnd - rowBegin)), dim3(256), 0, stream, ra);
+            e = hipGetLastError();
+            if (e != hipSuccess) return e;
+        }
     }
     return e;
 }

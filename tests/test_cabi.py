@@ -364,6 +364,24 @@ def test_swiglu_valid(aclnn):
     assert code == 0 and ws >= 16 * 256 * 4  # S workspace [M, N/2] fp32 plus tables
 
 
+def test_swiglu_workspace_is_capped(aclnn, monkeypatch):
+    """The fp32 SwiGLU workspace holds one band of rows: 512 MiB of it at most by default, whatever M is, and what
+    OPAPI_SWIGLU_WORKSPACE_MB says otherwise (never less than one tile of rows)."""
+    M, N = 1 << 20, 8192                                   # S for every row at once would be 16 GiB
+    tables = M * 4 * (N // 256) + (M // 32 + 8) * 16 + (1 << 16)   # row maxima per n-tile, m-tile table, header
+    code, ws = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=M, K=1024, N=N, E=8))
+    assert code == 0 and (512 << 20) - 256 * (N // 2) * 4 <= ws <= (512 << 20) + tables
+    monkeypatch.setenv("OPAPI_SWIGLU_WORKSPACE_MB", "64")
+    code, ws = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=M, K=1024, N=N, E=8))
+    assert code == 0 and (64 << 20) - 256 * (N // 2) * 4 <= ws <= (64 << 20) + tables
+    monkeypatch.setenv("OPAPI_SWIGLU_WORKSPACE_MB", "1")   # less than one tile of rows: one tile of rows it is
+    code, ws = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=4096, K=1024, N=28672, E=2))
+    assert code == 0 and ws >= 32 * (28672 // 2) * 4
+    small = _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=16, K=256, N=512, E=4))[1]
+    monkeypatch.delenv("OPAPI_SWIGLU_WORKSPACE_MB")
+    assert small == _status(aclnn, "aclnnGroupedMatmulSwigluQuant", _swiglu_args(aclnn, M=16, K=256, N=512, E=4))[1]
+
+
 @pytest.mark.parametrize("kw,fragment", [
     (dict(x_dtype=F16), "A8W8"),
     (dict(w_fmt=29), "storageShape for second input (weight) must be 5"),          # NZ format over plain 3-D storage

@@ -471,3 +471,41 @@ def test_pulled_tiles_swiglu_skewed(aclnn, oracle, dev, monkeypatch):
     diff = np.abs(q.cpu().numpy().astype(np.int32) - q_ref.astype(np.int32))
     assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
     np.testing.assert_allclose(qs.cpu().numpy(), qs_ref, rtol=1e-5)
+
+
+@pytest.mark.parametrize("cap_mb,K,N", [(1, 1024, 2048), (2, 1152, 2048), (1, 200, 768)])
+def test_swiglu_workspace_cap_runs_in_row_bands(aclnn, oracle, dev, monkeypatch, cap_mb, K, N):
+    """A cap on the fp32 SwiGLU workspace makes the operator run schedule, GEMM and requantisation once per band of rows
+    (band edges fall inside groups, at empty groups and past the list's last row).  Results are those of the single band,
+    bit for bit -- every row's accumulators, scale and maximum are its own -- and the workspace shrinks to the cap."""
+    rng = np.random.default_rng(1234 + K)
+    sizes = np.array([700, 3, 0, 0, 290, 31, 64, 65, 1, 257, 130, 0, 512, 90] + [int(v) for v in rng.integers(0, 40, 12)])
+    E = len(sizes)
+    cumsum = np.cumsum(sizes).astype(np.int64)
+    M = int(cumsum[-1]) + 37   # rows past the last group stay untouched
+    x = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, (E, N, K)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, (E, N)).astype(np.float32)
+    pt = rng.uniform(0.01, 0.1, M).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    args = (t(x), _weight_views(wt, dev, "kmajor"), t(cumsum), t(scale), t(pt))
+
+    def run():
+        q = torch.full((M, N // 2), 77, dtype=torch.int8, device=dev)
+        qs = torch.full((M,), -1.0, dtype=torch.float32, device=dev)
+        ws = aclnn.Workspace()
+        aclnn.grouped_matmul_swiglu_quant(*args, out=(q, qs), workspace=ws)
+        torch.cuda.synchronize()
+        return q.cpu().numpy(), qs.cpu().numpy(), ws.requested["aclnnGroupedMatmulSwigluQuant"]
+
+    q1, qs1, ws_one = run()
+    monkeypatch.setenv("OPAPI_SWIGLU_WORKSPACE_MB", str(cap_mb))
+    q2, qs2, ws_banded = run()
+    assert M * (N // 2) * 4 > 3 * (cap_mb << 20)          # at least three bands
+    assert ws_banded < ws_one and ws_banded <= (cap_mb << 20) + 256 * (N // 2) * 4 + M * 4 * (N // 128) + (1 << 16)
+    assert np.array_equal(q1, q2) and np.array_equal(qs1, qs2)
+    assert (q2[int(cumsum[-1]):] == 77).all() and (qs2[int(cumsum[-1]):] == -1.0).all()
+    q_ref, qs_ref = oracle.grouped_matmul_swiglu_quant(x[:int(cumsum[-1])], wt, scale, pt[:int(cumsum[-1])], cumsum, w_trans=True)
+    diff = np.abs(q2[:int(cumsum[-1])].astype(np.int32) - q_ref.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+    np.testing.assert_allclose(qs2[:int(cumsum[-1])], qs_ref, rtol=1e-5)
