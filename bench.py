@@ -19,7 +19,9 @@ the target is quoted on) behind the routing operator named by --routing (default
 rows and on the column of per-token scales), run eagerly.  The same line carries, under `other_configs`, a shorter
 measurement of the other halves of the metric: the decode shape c3 (eager and as a HIP-graph replay: HBM-bound), the
 Mixtral prefill shape c2 (the MFMA-bound one), the skewed shape c4, and c1 again as a graph replay and behind the other
-routing operator -- each with its ms per pass, per-kernel durations and both kernels' rooflines from the same timer.
+routing operator -- each with its ms per pass, per-kernel durations and both kernels' rooflines from the same timer
+(min(K, 20) passes each; ten times as many for the 0.4 ms decode pass, so that a block between two synchronisations is
+long against them -- with --config c3 give --steps 200 or more for the same reason).
 
 --calibration-copy appends, after the timed region, a few launches of the library's plain 1 GiB copy kernel: under
 `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` its counter readings give the factor that converts the counters to
@@ -309,9 +311,13 @@ def _other_configs(pkg, dev, headline, steps, warmup):
             continue
         release()
         w = Workload(pkg, pkg.synth.config(name), dev, routing=headline.ffn.routing)
-        out[name] = w.summary(w.measure(steps, warmup), steps, "eager two-phase calls")
+        # A decode pass is 0.4 ms: a block of four between two synchronisations would be timing the synchronisations
+        # (the first launch of a block has nothing to hide behind, the last wait is a host round trip: together ~0.1 ms).
+        # Ten times the passes make a block 16 ms.
+        n = steps * 10 if name == "c3" else steps
+        out[name] = w.summary(w.measure(n, warmup), n, "eager two-phase calls")
         if name == "c3":
-            out["c3_graph"] = w.summary(w.measure(steps, warmup, graph=True), steps,
+            out["c3_graph"] = w.summary(w.measure(n, warmup, graph=True), n,
                                         "HIP graph replay (kernel durations from eager passes)")
         del w
     release()
