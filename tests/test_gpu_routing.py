@@ -398,3 +398,37 @@ def test_four_byte_rows_are_copied_by_the_sort(aclnn, oracle, dev, T, K, E, acti
     ex_r, ri_r, cnt_r, _ = oracle.moe_init_routing_v2(x, idx, active_num=active, expert_num=E, count_flag=1)
     assert np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r)
     assert ex.shape == ex_r.shape and np.array_equal(ex.view(np.uint8), ex_r.view(np.uint8))
+
+
+# ------------------------------------------------------------------------------------------------ sort and gather in one launch
+@pytest.mark.parametrize("T,K,E,H,dtype", [
+    (1, 1, 4, 16, np.int8),            # one token, one 16-byte packet
+    (5, 3, 7, 48, np.int8),            # three packets per row, destinations shared out over thread groups
+    (64, 8, 128, 7168, np.int8),       # DeepSeek-V3 row width
+    (64, 64, 128, 32, np.float16),     # as many ids per token as the kernel caches
+    (256, 2, 512, 4096, np.int8),      # the most tokens (one workgroup each) and the most digit values
+    (256, 8, 16, 20480, np.float32),   # rows longer than the workgroup has threads for (81920 bytes = 5120 packets)
+    (257, 2, 8, 64, np.int8),          # one token more: one-workgroup sort, then the row gather
+    (100, 65, 8, 16, np.int8),         # one id per token more than cached: the same
+    (64, 8, 128, 24, np.int8),         # rows not a multiple of 16 bytes: the same
+])
+def test_decode_sized_calls_sort_and_gather_in_one_launch(aclnn, oracle, dev, T, K, E, H, dtype):
+    """Up to 256 tokens whose rows are whole 16-byte packets take one kernel for sort and row gather; the cases either side
+    of each limit take the separate kernels.  V2 with and without activeNum, V3 with scales and an expert sub-range."""
+    rng = np.random.default_rng(T * 131 + K * 7 + H)
+    x = (rng.standard_normal((T, H)) * 50).astype(dtype)
+    idx = rng.integers(0, E, (T, K)).astype(np.int32)
+    for active in (0, max(1, T * K // 3)):
+        for flag in (1, 2):
+            ex, ri, cnt, _ = _run(aclnn, dev, x, idx, active_num=active, expert_num=E, expert_tokens_count_or_cumsum_flag=flag)
+            ex_r, ri_r, cnt_r, _ = oracle.moe_init_routing_v2(x, idx, active_num=active, expert_num=E, count_flag=flag)
+            assert np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r)
+            assert ex.shape == ex_r.shape and np.array_equal(ex.view(np.uint8), ex_r.view(np.uint8))
+    scale = rng.random(T).astype(np.float32)
+    for rng_ in (None, (E // 4, max(E // 4 + 1, 3 * E // 4))):
+        for row_idx_type in (1, 0):
+            ex, ri, cnt, es = _run_v3(aclnn, dev, x, idx, scale, expert_num=E, expert_tokens_num_type=1,
+                                      active_expert_range=rng_, row_idx_type=row_idx_type)
+            ex_r, ri_r, cnt_r, es_r = oracle.moe_init_routing_v3(x, idx, scale, E, rng_, 1, row_idx_type)
+            assert np.array_equal(ri, ri_r) and np.array_equal(cnt, cnt_r) and np.array_equal(es, es_r)
+            assert np.array_equal(ex.view(np.uint8), ex_r.view(np.uint8))
