@@ -374,6 +374,9 @@ Plan MakePlan(const Problem& p) {
         for (int s : kShapes) {
             if (static_cast<double>(s) >= want) { plan.tileM = s; break; }
         }
+        // A handful of rows per group (decode): the 64-row shape, whose eight waves keep more of the weight stream in
+        // flight than the four of the 32-row shape (measured 0.3 - 0.7 % faster on both GEMMs of a 64-token step).
+        if (plan.tileM < 64) plan.tileM = 64;
         // tuning override: OPAPI_GEMM_TILE_M=<one of the shapes above>
         if (const char* env = std::getenv("OPAPI_GEMM_TILE_M")) {
             const int forced = std::atoi(env);
