@@ -807,13 +807,22 @@ __device__ __forceinline__ void StreamGemmBody(const KernelArgs& a, const int32_
     // instruction of slot q in the stage's list (activation part, then weight part)
     auto slotInstr = [&](int q) __attribute__((always_inline)) { return min(wave + q * Cfg::kWaves, Cfg::kInstr - 1); };
 
+    // 256-row tiles (the matrix-bound shapes): the tile's two base pointers are moved into scalar registers once per tile,
+    // and every slot of a stage is of the same part (activation / weight) in every wave.  A DMA then costs three
+    // instructions (LDS address, m0, the load) instead of nine (a select, a 64-bit vector add and two v_readfirstlane
+    // on top): the burst of refill requests behind a step's barrier, under which the matrix pipe has little to run, is a
+    // third as long.  Same-box A/B: Mixtral prefill gate/up 3.66 -> 3.56 ms, down 1.70 -> 1.67; the 192-row tiles of
+    // the HBM-bound shape measured 1.2 % slower with it and keep the vector form.
+    constexpr bool kScalarIssue = kTileM >= 256;
+    auto scalarBase = [&](const char* p) __attribute__((always_inline)) { return kScalarIssue ? UniformPtr(p) : p; };
+
     // The lambdas below are forced inline: left to the inliner's size heuristics, one of them staying a real call puts
     // the whole issue state (captured by reference) into scratch memory and the kernel runs three times slower.
     // Bases and lane offsets of the given part(s) for tile t.
     auto setupIssue = [&](const TileInfo& t, auto partsTag) __attribute__((always_inline)) {
         constexpr int kParts = decltype(partsTag)::value;
-        if (kParts & kPartA) issBaseA = reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(t.rowBase) * a.K;
-        if (kParts & kPartB) issBaseB = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(t.group) * a.wGroupStride;
+        if (kParts & kPartA) issBaseA = scalarBase(reinterpret_cast<const char*>(a.x) + static_cast<int64_t>(t.rowBase) * a.K);
+        if (kParts & kPartB) issBaseB = scalarBase(reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(t.group) * a.wGroupStride);
         // lane -> (row inside the instruction, LDS chunk slot); the global chunk it fetches is the one LdsOffset puts there
         const int lane = Opaque(tid & 63);
         const int rowIn = lane / Cfg::kChunksPerRow;
@@ -881,7 +890,7 @@ __device__ __forceinline__ void StreamGemmBody(const KernelArgs& a, const int32_
             } else if (!drained) {
                 drained = true;
                 // any mapped, 16-byte aligned kilobyte will do: the start of the last tile's expert's weights
-                const char* const hot = reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(tile.group) * a.wGroupStride;
+                const char* const hot = scalarBase(reinterpret_cast<const char*>(a.w) + static_cast<int64_t>(tile.group) * a.wGroupStride);
                 if (kParts & kPartA) issBaseA = hot;
                 if (kParts & kPartB) issBaseB = hot;
 #pragma unroll
@@ -917,7 +926,9 @@ __device__ __forceinline__ void StreamGemmBody(const KernelArgs& a, const int32_
         for (int q = 0; q < Cfg::kMaxPerWave; ++q) {
             if (kParts != kBothParts && (q < Cfg::kSlotsA) != (kParts == kPartA)) continue;
             const int g = slotInstr(q);
-            const bool isA = g < Cfg::kInstrA;
+            // where the activation instructions divide evenly among the waves, slot q is of the same part in every wave
+            constexpr bool kStaticSplit = kScalarIssue && Cfg::kInstrA % Cfg::kWaves == 0;
+            const bool isA = kStaticSplit ? q < Cfg::kInstrA / Cfg::kWaves : g < Cfg::kInstrA;
             // wave-uniform choice: activation rows always stay cacheable (the n-tiles of a group re-read them from L2);
             // on small tiles (every weight byte is used exactly once) the weights stream past the caches.  On large
             // tiles the m-tiles of a group share their weight columns through L2 and must not.
